@@ -26,6 +26,10 @@ def get_model(cfg: ModelConfig):
         from .kezunex import KezunexForCausalLM
 
         return KezunexForCausalLM(cfg)
+    if cfg.architecture == "relerax":
+        from .relerax import ReleraxForCausalLM
+
+        return ReleraxForCausalLM(cfg)
     raise ValueError(f"Unsupported architecture: {cfg.architecture}")
 
 
@@ -39,4 +43,8 @@ def native_extensions(cfg: ModelConfig) -> list[str]:
         from .kezunex import native_extensions as kz
 
         return kz(cfg)
+    if cfg.architecture == "relerax":
+        from .relerax import native_extensions as rx
+
+        return rx(cfg)
     return ["_C"]

@@ -25,6 +25,16 @@ that another design can assemble them differently:
 - ``MLSTMMixer``        matrix memory with exponential gating
 - ``ParallelMixer``     two mixers fed one input through a single merged
                         projection, their outputs mixed with fixed scales
+- ``scaled_rotary_frequencies``  rotation frequencies with the ramped
+                        (YaRN-style) stretch of the slowly turning pairs
+- ``RotatedAttention``  grouped-query softmax attention with rotated queries
+                        and keys (half-split or interleaved pairs), an optional
+                        sliding window, an optional sink in the softmax
+                        denominator, values that may be the unrotated keys, and
+                        an optional sigmoid output gate
+- ``BiasedDenseMLP``    down(act(up h + b) ) + b with a squared relu
+- ``RoutedExperts``     softmax router with a choice correction, top-k of
+                        small squared-relu experts plus identity experts
 
 The recurrent mixers keep their state (f32) and the last inputs of their short
 convolutions in per-sequence slots; a sequence that starts in a step starts
@@ -86,6 +96,40 @@ class ShortConv(nn.Module):
             meta.state_slots, add_input=True)
 
 
+def scaled_rotary_frequencies(base: float, dims: int,
+                              scaling: Optional[dict] = None) -> tuple[list, float]:
+    """Frequencies of the dims/2 rotated pairs, f_i = base^(-2i/dims), and the
+    factor that multiplies cos and sin (1 without scaling).
+
+    ``scaling`` = {factor s, original L, fast, slow} stretches the context by s
+    the YaRN way: pair i makes L f_i / 2 pi turns over the original length; the
+    pair index at which that count equals t is p(t) = dims ln(L / (2 pi t)) /
+    (2 ln base).  With lo = max(floor(p(fast)), 0), hi = min(ceil(p(slow)),
+    dims - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1) the
+    frequency becomes f_i / s * ramp_i + f_i * (1 - ramp_i): fast pairs keep
+    their frequency, slow pairs are interpolated.  cos and sin are multiplied
+    by 0.1 ln(s) + 1.  All of it in float64; callers round once to f32."""
+    import math
+
+    half = dims // 2
+    freqs = [float(base) ** (-2.0 * i / dims) for i in range(half)]
+    if not scaling:
+        return freqs, 1.0
+    s = float(scaling["factor"])
+    orig = float(scaling["original"])
+
+    def pair_at(turns: float) -> float:
+        return dims * math.log(orig / (2.0 * math.pi * turns)) / (2.0 * math.log(float(base)))
+
+    lo = max(math.floor(pair_at(float(scaling["fast"]))), 0)
+    hi = min(math.ceil(pair_at(float(scaling["slow"]))), dims - 1)
+    out = []
+    for i, f in enumerate(freqs):
+        ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+        out.append(f / s * ramp + f * (1.0 - ramp))
+    return out, 0.1 * math.log(s) + 1.0
+
+
 class LatentAttention(nn.Module):
     """Attention over a cached latent.
 
@@ -104,7 +148,11 @@ class LatentAttention(nn.Module):
     def __init__(self, width: int, *, heads: int, dim: int, rot_dim: int, vdim: int,
                  rank: int, scale: float, window: int, rot_base: float,
                  rot_dims: int, eps: float, kv_owner: bool, has_sink: bool,
-                 dtype: torch.dtype):
+                 dtype: torch.dtype, rot_interleaved: bool = False,
+                 rot_scaling: Optional[dict] = None, head_gate: bool = False):
+        """``rot_interleaved``: dim 2i is paired with 2i+1 instead of i with
+        i + rot_dims/2.  ``rot_scaling``: see ``scaled_rotary_frequencies``.
+        ``head_gate``: head h's output is multiplied by sigmoid(W_g x)_h."""
         super().__init__()
         tp = get_tp_world_size()
         self.heads = divide(heads, tp)
@@ -129,17 +177,23 @@ class LatentAttention(nn.Module):
             torch.empty(self.heads, rank, vdim, dtype=dtype).normal_(0.0, 0.02),
             requires_grad=False)
         self.sink = _f32_param(self.heads) if has_sink else None
-        half = rot_dims // 2
-        inv_freq = torch.tensor(
-            [float(rot_base) ** (-2.0 * i / rot_dims) for i in range(half)],
-            dtype=torch.float64).to(torch.float32)
-        self.register_buffer("inv_freq", inv_freq, persistent=False)
+        self.rot_interleaved = rot_interleaved
+        freqs, self.rot_mag = scaled_rotary_frequencies(rot_base, rot_dims, rot_scaling)
+        self.register_buffer(
+            "inv_freq", torch.tensor(freqs, dtype=torch.float64).to(torch.float32),
+            persistent=False)
+        # this rank's heads' rows of the gate projection
+        self.gate_weight = (
+            nn.Parameter(torch.empty(self.heads, width, dtype=dtype).normal_(0.0, 0.02),
+                         requires_grad=False) if head_gate else None)
 
     # -- weights -----------------------------------------------------------
-    def load(self, q, dkv, dkv_norm, uk, uv, sink, o) -> None:
+    def load(self, q, dkv, dkv_norm, uk, uv, sink, o, gate=None) -> None:
         r, h = get_tp_rank(), self.heads
         self.q_proj.load_full_weight(q)
         self.o_proj.load_full_weight(o)
+        if self.gate_weight is not None:
+            self.gate_weight.data.copy_(gate[r * h:(r + 1) * h].to(self.dtype))
         if self.kv_owner:
             self.dkv_weight.data.copy_(dkv.to(self.dtype))
             self.dkv_norm.data.copy_(dkv_norm.float())
@@ -156,12 +210,13 @@ class LatentAttention(nn.Module):
         t = h.shape[0]
         nh, d, r, rank = self.heads, self.dim, self.rot_dim, self.rank
         q = self.q_proj(h).view(t, nh, d + r)
-        ops.rope_partial(q, positions, self.inv_freq, d, self.rot_dims)
+        ops.rope_partial(q, positions, self.inv_freq, d, self.rot_dims,
+                         self.rot_interleaved, self.rot_mag)
         if self.kv_owner:
             dkv = ops.linear(h, self.dkv_weight)
             ops.latent_kv_write(dkv, self.dkv_norm, self.eps, positions,
                                 self.inv_freq, self.rot_dims, cache,
-                                meta.slot_mapping)
+                                meta.slot_mapping, self.rot_interleaved, self.rot_mag)
         # fold the unrotated query into latent space: [H, T, rank]
         q_lat = torch.bmm(q[:, :, :d].transpose(0, 1), self.uk).transpose(0, 1)
         q_rot = q[:, :, d:]
@@ -180,6 +235,10 @@ class LatentAttention(nn.Module):
                 meta.decode_seq_lens, self.scale, self.window, self.sink,
                 out=o_view[npt:])
         o = torch.bmm(o_lat, self.uv_t)                    # [H, T, vdim]
+        if self.gate_weight is not None:
+            # gate and the [H, T] -> [T, H] regrouping in one pass
+            g = ops.linear(h, self.gate_weight)            # [T, H]
+            return self.o_proj(ops.sigmoid_gate_mul(o.transpose(0, 1), g))
         return self.o_proj(o.transpose(0, 1).reshape(t, nh * self.vdim))
 
 
@@ -588,3 +647,191 @@ class ParallelMixer(nn.Module):
         b = ops.linear(self.right.mix(proj[:, n:], positions, cache[nl:], meta),
                        self.right.o_weight)
         return a, b
+
+
+class RotatedAttention(_Mixer):
+    """Causal grouped-query softmax attention with rotary positions.
+
+    Projected rows: [q | k | v? | gate?].  The first ``rot_dims`` dims of every
+    query and key head are rotated (pairs (i, i + rot_dims/2), or (2i, 2i+1)
+    when ``rot_interleaved``); score = q . k * scale; a query at position i
+    sees keys j with 0 <= i - j < window (window 0: every j <= i); with
+    ``sink`` (a logit) the softmax denominator also holds exp(sink), a key
+    that has no value.  ``values_from_keys``: there is no value projection,
+    the values are the keys as projected, before rotation (vdim = dim).
+    ``gate`` "elementwise": the concatenated heads are multiplied by
+    sigmoid(W_g h) before the output projection."""
+
+    def __init__(self, width: int, *, heads: int, kv_heads: int, dim: int, vdim: int,
+                 scale: float, window: int = 0, sink: Optional[float] = None,
+                 rot_base: float = 10000.0, rot_dims: int = 0,
+                 rot_interleaved: bool = False, rot_scaling: Optional[dict] = None,
+                 values_from_keys: bool = False, gate: Optional[str] = None,
+                 own_in: bool = True, dtype: torch.dtype = torch.bfloat16):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        if values_from_keys and vdim != dim:
+            raise ValueError("values taken from the keys have the key size")
+        if gate not in (None, "elementwise"):
+            raise ValueError(f"unknown gate {gate!r}")
+        if rot_dims % 2 or rot_dims > dim:
+            raise ValueError("rot_dims must be even and at most dim")
+        self.heads, self.kv_heads, self.dim, self.vdim = heads, kv_heads, dim, vdim
+        self.scale, self.window, self.sink = scale, window, sink
+        self.rot_dims, self.rot_interleaved = rot_dims, rot_interleaved
+        self.values_from_keys, self.gate = values_from_keys, gate
+        self.in_rows = (heads * dim + kv_heads * dim
+                        + (0 if values_from_keys else kv_heads * vdim)
+                        + (heads * vdim if gate else 0))
+        self.out_rows = heads * vdim
+        self._alloc(width, own_in, dtype)
+        freqs, self.rot_mag = scaled_rotary_frequencies(rot_base, max(rot_dims, 2), rot_scaling)
+        self.register_buffer(
+            "inv_freq", torch.tensor(freqs, dtype=torch.float64).to(torch.float32),
+            persistent=False)
+
+    def load_in(self, weight, bias, t) -> None:
+        off = 0
+        names = ["q", "k"] + ([] if self.values_from_keys else ["v"]) + (["g"] if self.gate else [])
+        for name in names:
+            n = t[name].shape[0]
+            weight[off:off + n].copy_(t[name].to(weight.dtype))
+            off += n
+        if off != self.in_rows:
+            raise ValueError("projection tensors do not add up to the mixer's rows")
+
+    def cache_shapes(self, block_size: int) -> list:
+        return [("paged", (block_size, self.kv_heads, self.dim), self.dtype),
+                ("paged", (block_size, self.kv_heads, self.vdim), self.dtype)]
+
+    def mix(self, proj, positions, cache, meta: AttnMetadata) -> torch.Tensor:
+        t = proj.shape[0]
+        nh, ng, d, dv = self.heads, self.kv_heads, self.dim, self.vdim
+        a = nh * d
+        b = a + ng * d
+        k_cache, v_cache = cache
+        k = proj[:, a:b].view(t, ng, d)
+        if self.values_from_keys:
+            v, c = k, b
+        else:
+            c = b + ng * dv
+            v = proj[:, b:c].view(t, ng, dv)
+        q = ops.rope_kv_cache_write(
+            proj[:, :a].view(t, nh, d), k, v, positions, self.inv_freq, self.rot_dims,
+            self.rot_interleaved, self.rot_mag, k_cache, v_cache, meta.slot_mapping)
+        out = torch.empty((t, nh, dv), dtype=proj.dtype, device=proj.device)
+        npt = meta.num_prefill_tokens
+        if npt:
+            ops.gqa_attention_prefill(
+                q[:npt], k_cache, v_cache, meta.prefill_block_tables,
+                meta.prefill_query_start_loc, meta.prefill_seq_lens, self.scale,
+                meta.max_prefill_query_len, out=out[:npt], window=self.window,
+                sink=self.sink)
+        if meta.num_decode_seqs:
+            ops.gqa_attention_decode(
+                q[npt:], k_cache, v_cache, meta.decode_block_tables,
+                meta.decode_seq_lens, self.scale, out=out[npt:], window=self.window,
+                sink=self.sink)
+        if self.gate:
+            return ops.sigmoid_gate_mul(out, proj[:, c:].view(t, nh, dv))
+        return out.view(t, nh * dv)
+
+
+class BiasedDenseMLP(nn.Module):
+    """down(relu(up h + b_up)^2) + b_down."""
+
+    def __init__(self, width: int, ff: int, dtype: torch.dtype):
+        super().__init__()
+        if get_tp_world_size() != 1:
+            raise ValueError("BiasedDenseMLP is not sharded; run it with one rank")
+        self.up = _randn_param((ff, width), dtype, std=width ** -0.5)
+        self.up_bias = nn.Parameter(torch.zeros(ff, dtype=dtype), requires_grad=False)
+        self.down = _randn_param((width, ff), dtype, std=ff ** -0.5)
+        self.down_bias = nn.Parameter(torch.zeros(width, dtype=dtype), requires_grad=False)
+
+    def load(self, up, up_b, down, down_b) -> None:
+        for p, t in ((self.up, up), (self.up_bias, up_b), (self.down, down),
+                     (self.down_bias, down_b)):
+            p.data.copy_(t.to(p.dtype))
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        a = ops.relu2(ops.linear(h, self.up), self.up_bias)
+        return ops.linear(a, self.down, self.down_bias)
+
+
+class RoutedExperts(nn.Module):
+    """Mixture of ``experts`` small feed-forwards down(relu(up h)^2) (no
+    biases) and ``identity`` experts that return their input.
+
+    Router: z = W_r h in f32, s = softmax(z) over all experts + identity; the
+    ``top`` largest s + correction are chosen; weights = their s, divided by
+    their sum (+ 1e-20).  Returns (y, identity weight [T] f32): y is the
+    weighted sum of the chosen real experts, the identity share is left to the
+    caller's residual kernel (h times the returned per-row weight).
+
+    Two ways to run the experts, chosen by shape at construction:
+
+    - stacked: one product with all experts' up-projections stacked
+      [E * ff, width], the squared relu times the row's weight of the column's
+      expert (0 where the expert was not chosen), one product with the
+      down-projections stacked along the contraction axis [width, E * ff] —
+      the zeros make the unchosen experts vanish exactly.  Any size, f32 or
+      bf16, no sorting, shape-static; costs E / top of the chosen experts'
+      multiply-adds, so it is the path for few or small experts.
+    - grouped: token-expert pairs sorted by expert, one grouped product per
+      projection over the expert segments (bf16, sizes in multiples of 128)."""
+
+    def __init__(self, width: int, *, experts: int, identity: int, top: int, ff: int,
+                 dtype: torch.dtype, grouped: Optional[bool] = None):
+        super().__init__()
+        if get_tp_world_size() != 1:
+            raise ValueError("RoutedExperts is not sharded; run it with one rank")
+        if not 1 <= top <= experts + identity:
+            raise ValueError("top must lie between 1 and the number of router outputs")
+        self.width, self.experts, self.identity, self.top, self.ff = width, experts, identity, top, ff
+        self.dtype = dtype
+        fits = dtype == torch.bfloat16 and ff % 128 == 0 and width % 128 == 0
+        self.grouped = (fits and experts > 2 * top) if grouped is None else bool(grouped)
+        if self.grouped and not fits:
+            raise ValueError("grouped experts need bf16 and sizes in multiples of 128")
+        self.router = nn.Parameter(
+            torch.empty(experts + identity, width, dtype=torch.float32).normal_(0.0, width ** -0.5),
+            requires_grad=False)
+        self.correction = _f32_param(experts + identity)
+        self.up = _randn_param((experts, ff, width), dtype, std=width ** -0.5)
+        if self.grouped:
+            self.down = _randn_param((experts, width, ff), dtype, std=ff ** -0.5)
+        else:
+            self.down = _randn_param((width, experts * ff), dtype, std=ff ** -0.5)
+
+    def load(self, router, correction, ups: list, downs: list) -> None:
+        self.router.data.copy_(router.float())
+        self.correction.data.copy_(correction.float())
+        for e, (u, d) in enumerate(zip(ups, downs)):
+            self.up.data[e].copy_(u.to(self.dtype))
+            if self.grouped:
+                self.down.data[e].copy_(d.to(self.dtype))
+            else:
+                self.down.data[:, e * self.ff:(e + 1) * self.ff].copy_(d.to(self.dtype))
+
+    def forward(self, h: torch.Tensor):
+        z = torch.nn.functional.linear(h.float(), self.router)
+        dense, ident, ids, w = ops.moe_route(z, self.correction, self.top, self.experts)
+        if not self.grouped:
+            u = ops.linear(h, self.up.view(self.experts * self.ff, self.width))
+            return ops.linear(ops.relu2(u, None, dense), self.down), ident
+        t, top, ne = h.shape[0], self.top, self.experts
+        # pairs sorted by expert (identity experts sort last and are skipped)
+        flat = ids.reshape(-1).long()
+        order = torch.argsort(flat, stable=True)
+        pos = torch.empty_like(order)
+        pos[order] = torch.arange(t * top, device=h.device)
+        counts = torch.zeros(ne + self.identity, dtype=torch.int32, device=h.device)
+        counts.scatter_add_(0, flat, torch.ones_like(flat, dtype=torch.int32))
+        seg = torch.zeros(ne + 1, dtype=torch.int32, device=h.device)
+        seg[1:] = counts[:ne].cumsum(0).to(torch.int32)
+        xs = h[torch.div(order, top, rounding_mode="floor")]
+        a = ops.moe_gemm(xs, self.up, seg, gated=False, act="relu2")
+        ye = ops.moe_gemm(a, self.down, seg, gated=False)
+        return ops.moe_combine(ye, pos.view(t, top).to(torch.int32), ids, w, ne), ident

@@ -378,12 +378,19 @@ def moe_gemm(
     w: torch.Tensor,        # [E, 2N, K] (gated) or [E, N, K]
     seg_off: torch.Tensor,  # [E+1] int32 device row offsets
     gated: bool,
+    act: str | None = None,
 ) -> torch.Tensor:
-    """Grouped GEMM over expert segments (E16); gated fuses SiLU(g)*u."""
-    assert _native(x)
+    """Grouped GEMM over expert segments (E16); gated fuses SiLU(g)*u; a plain
+    product may be followed by ``act`` ("relu2": the squared relu).  Rows past
+    the last segment are left unwritten."""
+    if act not in (None, "relu2") or (gated and act):
+        raise ValueError(f"unknown activation {act!r}")
     n = w.shape[1] // 2 if gated else w.shape[1]
+    if x.device.type != "cuda" or _FORCE_REFERENCE:
+        return reference.moe_gemm(x, w, seg_off.cpu(), gated, act)
+    ext = _C if _C is not None else (_S if _native_seq(x) else None)
     out = torch.empty((x.shape[0], n), dtype=x.dtype, device=x.device)
-    _C.moe_gemm(out, x, w, seg_off, gated)
+    ext.moe_gemm(out, x, w, seg_off, 1 if gated else (2 if act == "relu2" else 0))
     return out
 
 
@@ -606,25 +613,30 @@ def causal_conv_state(h, weight, state, seq_start_loc, seq_lens, state_slots,
 
 
 def rope_partial(x: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor,
-                 offset: int, rot_dims: int) -> None:
-    """In place half-split rotation of dims [offset, offset+rot_dims) of every
-    head of x [T, H, D]; f32 angles position * inv_freq[i]."""
+                 offset: int, rot_dims: int, interleaved: bool = False,
+                 mag: float = 1.0) -> None:
+    """In place rotation of dims [offset, offset+rot_dims) of every head of
+    x [T, H, D]: dim i paired with i + rot_dims/2, or (``interleaved``) dim 2i
+    with 2i+1; f32 angles position * inv_freq[i], cos and sin times ``mag``."""
     if x.numel() and _native_seq(x):
-        _S.rope_partial(x, positions, inv_freq, int(offset), int(rot_dims))
+        _S.rope_partial(x, positions, inv_freq, int(offset), int(rot_dims),
+                        bool(interleaved), float(mag))
         return
-    reference.rope_partial(x, positions, inv_freq, offset, rot_dims)
+    reference.rope_partial(x, positions, inv_freq, offset, rot_dims, interleaved, mag)
 
 
 def latent_kv_write(dkv, norm_weight, eps, positions, inv_freq, rot_dims,
-                    cache, slot_mapping) -> None:
+                    cache, slot_mapping, interleaved: bool = False,
+                    mag: float = 1.0) -> None:
     """RMS-norm the latent part, rotate the shared key part, store the row in
-    the paged latent cache."""
+    the paged latent cache.  ``dkv`` may be a column slice of a wider matrix."""
     if dkv.numel() and _native_seq(dkv):
         _S.latent_kv_write(dkv, norm_weight, float(eps), positions, inv_freq,
-                           int(rot_dims), cache, slot_mapping)
+                           int(rot_dims), cache, slot_mapping, bool(interleaved),
+                           float(mag))
         return
     reference.latent_kv_write(dkv, norm_weight, eps, positions, inv_freq,
-                              rot_dims, cache, slot_mapping)
+                              rot_dims, cache, slot_mapping, interleaved, mag)
 
 
 def latent_attention_prefill(q_lat, q_rot, cache, block_tables, query_start_loc,
@@ -739,6 +751,12 @@ def _matrix_core_attention_fits(q: torch.Tensor, k_cache: torch.Tensor,
             and q.shape[1] == group * k_cache.shape[2])
 
 
+def _windowed_matrix_core_fits(q: torch.Tensor, k_cache: torch.Tensor,
+                               v_cache: torch.Tensor) -> bool:
+    """No matrix-core kernel takes a window or a sink yet."""
+    return False
+
+
 def attention_uses_matrix_cores(dtype: torch.dtype, heads: int, kv_heads: int,
                                 dim: int, vdim: int) -> bool:
     """Shape test of the above without tensors (which extensions a model needs)."""
@@ -747,12 +765,27 @@ def attention_uses_matrix_cores(dtype: torch.dtype, heads: int, kv_heads: int,
 
 
 def gqa_attention_prefill(q, k_cache, v_cache, block_tables, query_start_loc,
-                          seq_lens, scale, max_query_len, out: torch.Tensor) -> torch.Tensor:
+                          seq_lens, scale, max_query_len, out: torch.Tensor,
+                          window: int = 0, sink: float | None = None) -> torch.Tensor:
     """Causal grouped-query softmax attention of query chunks (the tail rows
     of each sequence) over the paged cache; q [T, H, dim], out [T, H, vdim].
+    ``window`` > 0: position i sees j with 0 <= i - j < window.  ``sink``: the
+    softmax denominator also holds exp(sink), a key without a value.
     bf16 shapes the MFMA kernels take run there, everything else (f32, other
     sizes, value size unlike the key size) on the any-shape kernel."""
     if q.numel() and _native_seq(q):
+        if window > 0 or sink is not None:
+            if _windowed_matrix_core_fits(q, k_cache, v_cache):
+                _S.windowed_attention_mfma(out, q, k_cache, v_cache, block_tables,
+                                           query_start_loc, seq_lens, float(scale),
+                                           int(max_query_len), int(window),
+                                           sink is not None, float(sink or 0.0))
+                return out
+            _S.paged_attention_any(out, q, k_cache, v_cache, block_tables,
+                                   query_start_loc, seq_lens, float(scale),
+                                   int(max_query_len), int(window),
+                                   sink is not None, float(sink or 0.0))
+            return out
         if _matrix_core_attention_fits(q, k_cache, v_cache):
             dst = out if out.is_contiguous() else torch.empty_like(q)
             _attn_ext().paged_attention_prefill(dst, q, k_cache, v_cache, block_tables,
@@ -763,19 +796,31 @@ def gqa_attention_prefill(q, k_cache, v_cache, block_tables, query_start_loc,
             return out
         _S.paged_attention_any(out, q, k_cache, v_cache, block_tables,
                                query_start_loc, seq_lens, float(scale),
-                               int(max_query_len))
+                               int(max_query_len), 0, False, 0.0)
         return out
     out.copy_(reference.paged_attention(
         q, k_cache, v_cache, block_tables.cpu(), query_start_loc.cpu(),
-        seq_lens.cpu(), scale))
+        seq_lens.cpu(), scale, window, sink))
     return out
 
 
 def gqa_attention_decode(q, k_cache, v_cache, block_tables, seq_lens, scale,
-                         out: torch.Tensor) -> torch.Tensor:
+                         out: torch.Tensor, window: int = 0,
+                         sink: float | None = None) -> torch.Tensor:
     """Same attention for one new query per sequence (seq_len 0 = padding row,
     zeros)."""
     if q.numel() and _native_seq(q):
+        if window > 0 or sink is not None:
+            if _windowed_matrix_core_fits(q, k_cache, v_cache):
+                _S.windowed_attention_mfma(out, q, k_cache, v_cache, block_tables,
+                                           None, seq_lens, float(scale), 1,
+                                           int(window), sink is not None,
+                                           float(sink or 0.0))
+                return out
+            _S.paged_attention_any(out, q, k_cache, v_cache, block_tables, None,
+                                   seq_lens, float(scale), 1, int(window),
+                                   sink is not None, float(sink or 0.0))
+            return out
         if _matrix_core_attention_fits(q, k_cache, v_cache):
             if out.is_contiguous():
                 _attn_ext().paged_attention_decode(out, q, k_cache, v_cache,
@@ -787,12 +832,13 @@ def gqa_attention_decode(q, k_cache, v_cache, block_tables, seq_lens, scale,
                 out.copy_(tmp)
             return out
         _S.paged_attention_any(out, q, k_cache, v_cache, block_tables, None,
-                               seq_lens, float(scale), 1)
+                               seq_lens, float(scale), 1, 0, False, 0.0)
         return out
     n = q.shape[0]
     qsl = torch.arange(n + 1, dtype=torch.int32)
     out.copy_(reference.paged_attention(
-        q, k_cache, v_cache, block_tables.cpu(), qsl, seq_lens.cpu(), scale))
+        q, k_cache, v_cache, block_tables.cpu(), qsl, seq_lens.cpu(), scale,
+        window, sink))
     return out
 
 
@@ -853,3 +899,95 @@ def mlstm_scan(q, k, v, i_pre, f_pre, i_bias, f_bias, cap, q_scale, s_state,
     return reference.mlstm_scan(q, k, v, i_pre, f_pre, i_bias, f_bias, cap, q_scale,
                                 s_state, n_state, m_state, seq_start_loc.cpu(),
                                 seq_lens.cpu(), state_slots.cpu())
+
+
+# ---------------------------------------------------------------------------
+# Two-norm parallel layers, rotated grouped-query attention whose cache is
+# written by one op, output gates, squared-relu feed-forwards, routed experts
+# with identity experts.  Same extension as the stream ops.
+# ---------------------------------------------------------------------------
+
+
+def stream_add_rms_norm_pair(x: torch.Tensor, a: torch.Tensor | None,
+                             b: torch.Tensor | None, w1: torch.Tensor | None,
+                             w2: torch.Tensor | None, eps: float,
+                             out_dtype: torch.dtype,
+                             row_scale: torch.Tensor | None = None,
+                             c: torch.Tensor | None = None):
+    """x (f32, in place) += a + b + row_scale[:, None] * c (each optional;
+    nothing is added when ``a`` is None), then the two RMS norms that read the
+    updated stream next, which share one statistic: x / sqrt(mean(x^2) + eps)
+    times w1 and times w2.  Returns (h1, h2), None where the weight is None."""
+    if x.numel() and _native_seq(x):
+        h1 = torch.empty(x.shape, dtype=out_dtype, device=x.device) if w1 is not None else None
+        h2 = torch.empty(x.shape, dtype=out_dtype, device=x.device) if w2 is not None else None
+        _S.stream_add_rms_norm_pair(x, a, b, row_scale, c, w1, w2, float(eps), h1, h2)
+        return h1, h2
+    return reference.stream_add_rms_norm_pair(x, a, b, row_scale, c, w1, w2, eps, out_dtype)
+
+
+def rope_kv_cache_write(q, k, v, positions, inv_freq, rot_dims: int, interleaved: bool,
+                        mag: float, k_cache, v_cache, slot_mapping) -> torch.Tensor:
+    """Rotate the first ``rot_dims`` dims of every head of q [T, H, dim] and
+    k [T, G, dim] (f32 angles position * inv_freq[i], cos and sin times
+    ``mag``), store rotated keys and v [T, G, vdim] as given in the paged cache.
+    q, k, v may be views into a merged projection (v may alias k: the values
+    are then the unrotated keys).  Returns contiguous rotated queries."""
+    if q.numel() and _native_seq(q):
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        _S.rope_kv_cache_write(out, q, k, v, positions, inv_freq, int(rot_dims),
+                               bool(interleaved), float(mag), k_cache, v_cache,
+                               slot_mapping)
+        return out
+    return reference.rope_kv_cache_write(q, k, v, positions, inv_freq, rot_dims,
+                                         interleaved, mag, k_cache, v_cache, slot_mapping)
+
+
+def sigmoid_gate_mul(o: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """o [T, H, D] (any head / row strides) times sigmoid(gate) with gate
+    [T, H, D] (elementwise) or [T, H] (one per head), f32 sigmoid; returns
+    contiguous [T, H * D]."""
+    if o.numel() and _native_seq(o):
+        t, h, d = o.shape
+        out = torch.empty((t, h * d), dtype=o.dtype, device=o.device)
+        _S.sigmoid_gate_mul(out, o, gate)
+        return out
+    return reference.sigmoid_gate_mul(o, gate)
+
+
+def relu2(x: torch.Tensor, bias: torch.Tensor | None = None,
+          col_scale: torch.Tensor | None = None) -> torch.Tensor:
+    """relu(x + bias)^2; with ``col_scale`` [T, E] f32 also times
+    col_scale[t, column // (columns / E)]."""
+    if x.numel() and _native_seq(x):
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        _S.relu2(out, x, bias, col_scale)
+        return out
+    return reference.relu2(x, bias, col_scale)
+
+
+def moe_route(logits: torch.Tensor, correction: torch.Tensor, top: int, num_real: int):
+    """Softmax router with a choice correction and identity experts; see
+    reference.moe_route.  Returns (dense [T, num_real] f32, identity [T] f32,
+    ids [T, top] int32, weights [T, top] f32)."""
+    if logits.numel() and _native_seq(logits):
+        t, n = logits.shape
+        dev = logits.device
+        dense = torch.empty((t, num_real), dtype=torch.float32, device=dev)
+        ident = torch.empty((t,), dtype=torch.float32, device=dev)
+        ids = torch.empty((t, top), dtype=torch.int32, device=dev)
+        w = torch.empty((t, top), dtype=torch.float32, device=dev)
+        _S.moe_route(dense, ident, ids, w, logits, correction, int(num_real))
+        return dense, ident, ids, w
+    return reference.moe_route(logits, correction, top, num_real)
+
+
+def moe_combine(ye: torch.Tensor, pos: torch.Tensor, ids: torch.Tensor,
+                weights: torch.Tensor, num_real: int) -> torch.Tensor:
+    """Weighted sum of each token's real-expert outputs, gathered from the
+    expert-sorted rows ``ye`` through ``pos`` [T, top]; no atomics."""
+    if ye.numel() and _native_seq(ye):
+        out = torch.empty((pos.shape[0], ye.shape[1]), dtype=ye.dtype, device=ye.device)
+        _S.moe_combine(out, ye, pos, ids, weights, int(num_real))
+        return out
+    return reference.moe_combine(ye, pos, ids, weights, num_real)

@@ -114,9 +114,13 @@ def paged_attention(
     query_start_loc: torch.Tensor,  # [num_seqs + 1] (cpu)
     seq_lens: torch.Tensor,         # [num_seqs] total context per seq (cpu)
     scale: float,
+    window: int = 0,
+    sink: float | None = None,
 ) -> torch.Tensor:
     """Causal paged attention over queries that are the *tail* of each
-    sequence (covers prefill chunks and single-token decode uniformly)."""
+    sequence (covers prefill chunks and single-token decode uniformly).
+    ``window`` > 0: a query at position i sees keys j with 0 <= i - j < window.
+    ``sink``: the softmax denominator also holds exp(sink) (no key, no value)."""
     num_heads = q.shape[1]
     num_kv_heads = k_cache.shape[2]
     group = num_heads // num_kv_heads
@@ -141,8 +145,15 @@ def paged_attention(
         kpos = torch.arange(seq_len, device=q.device)
         qpos = torch.arange(seq_len - q_len, seq_len, device=q.device)
         mask = kpos[None, :] > qpos[:, None]
+        if window > 0:
+            mask = mask | (qpos[:, None] - kpos[None, :] >= window)
         scores.masked_fill_(mask.unsqueeze(0), float("-inf"))
-        probs = torch.softmax(scores, dim=-1)
+        if sink is None:
+            probs = torch.softmax(scores, dim=-1)
+        else:
+            m = scores.max(dim=-1, keepdim=True).values.clamp(min=float(sink))
+            probs = torch.exp(scores - m)
+            probs = probs / (probs.sum(dim=-1, keepdim=True) + torch.exp(float(sink) - m))
         out[s:e] = torch.einsum("hqs,shd->qhd", probs, vf).to(q.dtype)
     return out
 
@@ -249,19 +260,29 @@ def causal_conv_state(
 
 
 def rope_partial(x: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor,
-                 offset: int, rot_dims: int) -> None:
+                 offset: int, rot_dims: int, interleaved: bool = False,
+                 mag: float = 1.0) -> None:
     """In place: dims [offset, offset+rot_dims) of the last axis of x [T, H, D]
-    are rotated, dim i paired with i + rot_dims/2, angle = position * inv_freq[i]
-    in f32."""
+    are rotated, dim i paired with i + rot_dims/2 (or, ``interleaved``, dim 2i
+    with 2i+1), angle = position * inv_freq[i] in f32; cos and sin are
+    multiplied by ``mag``."""
     half = rot_dims // 2
     ang = positions.to(torch.float32).unsqueeze(1) * inv_freq.float().unsqueeze(0)
     cos, sin = ang.cos().unsqueeze(1), ang.sin().unsqueeze(1)
-    u = x[..., offset:offset + half].float()
-    v = x[..., offset + half:offset + rot_dims].float()
+    if mag != 1.0:
+        cos, sin = cos * mag, sin * mag
+    if interleaved:
+        ia = slice(offset, offset + rot_dims, 2)
+        ib = slice(offset + 1, offset + rot_dims, 2)
+    else:
+        ia = slice(offset, offset + half)
+        ib = slice(offset + half, offset + rot_dims)
+    u = x[..., ia].float()
+    v = x[..., ib].float()
     a = (u * cos - v * sin).to(x.dtype)   # both halves before either store:
     b = (v * cos + u * sin).to(x.dtype)   # for f32 x, u and v alias x
-    x[..., offset:offset + half] = a
-    x[..., offset + half:offset + rot_dims] = b
+    x[..., ia] = a
+    x[..., ib] = b
 
 
 def latent_kv_write(
@@ -273,12 +294,14 @@ def latent_kv_write(
     rot_dims: int,
     cache: torch.Tensor,        # [blocks, block_size, rank + rot]
     slot_mapping: torch.Tensor,
+    interleaved: bool = False,
+    mag: float = 1.0,
 ) -> None:
     rank = norm_weight.shape[0]
     c = dkv[:, :rank].float()
     c = c * torch.rsqrt(c.pow(2).mean(dim=-1, keepdim=True) + eps) * norm_weight.float()
     kr = dkv[:, rank:].float().unsqueeze(1).clone()
-    rope_partial(kr, positions, inv_freq, 0, rot_dims)
+    rope_partial(kr, positions, inv_freq, 0, rot_dims, interleaved, mag)
     row = torch.cat([c, kr.squeeze(1)], dim=-1).to(cache.dtype)
     bs = cache.shape[1]
     ok = slot_mapping >= 0
@@ -566,3 +589,129 @@ def mlstm_scan(
             o[i] = torch.einsum("hvd,hd->hv", s, qf[i]) / den.view(heads, 1)
         s_state[slot], n_state[slot], m_state[slot] = s, n, m
     return o.view(t, heads * vdim)
+
+
+# ---------------------------------------------------------------------------
+# Two-norm parallel layers, rotated grouped-query attention whose cache is
+# written by one op, output gates, squared-relu feed-forwards, routed experts
+# with identity experts
+# ---------------------------------------------------------------------------
+
+
+def stream_add_rms_norm_pair(x: torch.Tensor, a: torch.Tensor | None,
+                             b: torch.Tensor | None, row_scale: torch.Tensor | None,
+                             c: torch.Tensor | None, w1: torch.Tensor | None,
+                             w2: torch.Tensor | None, eps: float,
+                             out_dtype: torch.dtype):
+    """x (f32, in place) += a + b + row_scale[:, None] * c (each optional), then
+    two RMS norms of the updated row that share one statistic:
+    x / sqrt(mean(x^2) + eps) * w1 and * w2.  Returns (h1, h2), None where the
+    weight is None."""
+    if a is not None:
+        s = a.float()
+        if b is not None:
+            s = s + b.float()
+        if c is not None:
+            s = s + row_scale.float().unsqueeze(1) * c.float()
+        x.add_(s)
+    if w1 is None and w2 is None:
+        return None, None
+    u = x * torch.rsqrt(x.pow(2).mean(dim=-1, keepdim=True) + eps)
+    h1 = (u * w1.float()).to(out_dtype) if w1 is not None else None
+    h2 = (u * w2.float()).to(out_dtype) if w2 is not None else None
+    return h1, h2
+
+
+def rope_kv_cache_write(q, k, v, positions, inv_freq, rot_dims: int, interleaved: bool,
+                        mag: float, k_cache, v_cache, slot_mapping) -> torch.Tensor:
+    """Rotate the first ``rot_dims`` dims of every head of q [T, H, dim] and
+    k [T, G, dim]; store rotated keys and v [T, G, vdim] (as given) in the paged
+    cache (slot < 0: skipped).  Returns contiguous rotated queries."""
+    qo = q.clone()
+    kr = k.clone()
+    if rot_dims:
+        rope_partial(qo, positions, inv_freq, 0, rot_dims, interleaved, mag)
+        rope_partial(kr, positions, inv_freq, 0, rot_dims, interleaved, mag)
+    bs = k_cache.shape[1]
+    ok = slot_mapping >= 0
+    sm = slot_mapping[ok]
+    blk, off = torch.div(sm, bs, rounding_mode="floor"), sm % bs
+    k_cache[blk, off] = kr[ok].to(k_cache.dtype)
+    v_cache[blk, off] = v[ok].to(v_cache.dtype)
+    return qo
+
+
+def sigmoid_gate_mul(o: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """o [T, H, D] (any strides) times sigmoid(gate), gate [T, H, D] (one per
+    element) or [T, H] (one per head); f32 sigmoid; returns contiguous
+    [T, H * D]."""
+    t, h, d = o.shape
+    g = torch.sigmoid(gate.float())
+    g = g.unsqueeze(-1) if gate.dim() == 2 else g
+    return (o.float() * g).to(o.dtype).reshape(t, h * d)
+
+
+def relu2(x: torch.Tensor, bias: torch.Tensor | None = None,
+          col_scale: torch.Tensor | None = None) -> torch.Tensor:
+    """relu(x + bias)^2, optionally times col_scale[t, column // (cols / E)]
+    (col_scale [T, E] f32: one factor per row and block of columns)."""
+    z = x.float()
+    if bias is not None:
+        z = z + bias.float()
+    z = torch.clamp(z, min=0.0)
+    z = z * z
+    if col_scale is not None:
+        e = col_scale.shape[1]
+        z = (z.view(z.shape[0], e, -1) * col_scale.float().unsqueeze(-1)).view(z.shape)
+    return z.to(x.dtype)
+
+
+def moe_route(logits: torch.Tensor, correction: torch.Tensor, top: int, num_real: int):
+    """Router of a mixture with identity experts.  logits [T, N] f32 over the
+    ``num_real`` real experts followed by N - num_real identity experts.
+    s = softmax(logits); the ``top`` experts with the largest s + correction
+    are chosen (ties: the lower index); weights = s[chosen] / (sum + 1e-20).
+    Returns (dense [T, num_real] f32: weight of each real expert or 0,
+    identity [T] f32: summed weight of the chosen identity experts,
+    ids [T, top] int32, weights [T, top] f32)."""
+    s = torch.softmax(logits.float(), dim=-1)
+    choice = s + correction.float()
+    # stable descending order: ties go to the lower index
+    order = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, :top]
+    w = torch.gather(s, 1, order)
+    w = w / (w.sum(dim=-1, keepdim=True) + 1e-20)
+    full = torch.zeros_like(s).scatter_(1, order, w)
+    return (full[:, :num_real].contiguous(), full[:, num_real:].sum(dim=-1),
+            order.to(torch.int32), w)
+
+
+def moe_combine(ye: torch.Tensor, pos: torch.Tensor, ids: torch.Tensor,
+                weights: torch.Tensor, num_real: int) -> torch.Tensor:
+    """out[t] = sum over k with ids[t, k] < num_real of weights[t, k] *
+    ye[pos[t, k]] (ye: expert outputs of the token-expert pairs sorted by
+    expert, pos [T, top]: where pair (t, k) went); f32 sums."""
+    rows = ye[pos.long().reshape(-1)].float().view(*pos.shape, -1)
+    w = torch.where(ids < num_real, weights.float(), torch.zeros_like(weights, dtype=torch.float32))
+    rows = torch.where((ids < num_real).unsqueeze(-1), rows, torch.zeros_like(rows))
+    return (rows * w.unsqueeze(-1)).sum(dim=1).to(ye.dtype)
+
+
+def moe_gemm(x: torch.Tensor, w: torch.Tensor, seg_off: torch.Tensor, gated: bool,
+             act: str | None = None) -> torch.Tensor:
+    """Rows seg_off[e] .. seg_off[e+1] of x times expert e's weight w[e]
+    ([2N, K] gated: silu(first half) * second half; else [N, K], optionally
+    followed by the squared relu).  Rows past the last segment are zeros."""
+    n = w.shape[1] // 2 if gated else w.shape[1]
+    out = torch.zeros((x.shape[0], n), dtype=x.dtype, device=x.device)
+    off = seg_off.tolist()
+    for e in range(w.shape[0]):
+        a, b = off[e], off[e + 1]
+        if b <= a:
+            continue
+        y = x[a:b].float() @ w[e].float().T
+        if gated:
+            y = torch.nn.functional.silu(y[:, :n]) * y[:, n:]
+        elif act == "relu2":
+            y = torch.clamp(y, min=0.0) ** 2
+        out[a:b] = y.to(x.dtype)
+    return out
