@@ -91,7 +91,7 @@ void launch_sample_argmax(long*, const T*, const float*, const float*, int,
                           int, hipStream_t);
 void launch_moe_gemm(__hip_bfloat16*, const __hip_bfloat16*,
                      const __hip_bfloat16*, const int*, int, int, int, int,
-                     bool, hipStream_t);
+                     int, hipStream_t);
 
 // paged attention (bindings_attn.cpp, shared with the `_C_attn` extension)
 void register_attention_ops(pybind11::module& m);
@@ -368,12 +368,15 @@ void lora_bgmv(torch::Tensor out, torch::Tensor x, torch::Tensor a_stack,
 }
 
 void moe_gemm(torch::Tensor y, torch::Tensor x, torch::Tensor w,
-              torch::Tensor seg_off, bool gated) {
+              torch::Tensor seg_off, int64_t mode) {
+  // mode 0: plain, 1: silu(first half) * second half, 2: squared relu
   const int T = x.size(0);
   const int K = x.size(1);
   const int E = w.size(0);
   const long wn = w.size(1);
+  const bool gated = mode == 1;
   const int N = gated ? (int)(wn / 2) : (int)wn;
+  TORCH_CHECK(mode >= 0 && mode <= 2);
   TORCH_CHECK(x.scalar_type() == at::ScalarType::BFloat16 &&
               w.scalar_type() == at::ScalarType::BFloat16 &&
               y.scalar_type() == at::ScalarType::BFloat16);
@@ -386,7 +389,7 @@ void moe_gemm(torch::Tensor y, torch::Tensor x, torch::Tensor w,
   launch_moe_gemm(reinterpret_cast<__hip_bfloat16*>(y.data_ptr()),
                   reinterpret_cast<const __hip_bfloat16*>(x.data_ptr()),
                   reinterpret_cast<const __hip_bfloat16*>(w.data_ptr()),
-                  seg_off.data_ptr<int>(), E, N, K, T, gated,
+                  seg_off.data_ptr<int>(), E, N, K, T, (int)mode,
                   current_stream());
 }
 

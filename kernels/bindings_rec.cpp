@@ -28,8 +28,8 @@ void launch_qk_norm_cache_write(T*, const T*, long, const T*, long, const T*,
 template <typename T>
 void launch_paged_attention_any(T*, long, const T*, long, const T*, const T*,
                                 const int*, int, const int*, const int*, int,
-                                float, int, int, int, int, int, int, int,
-                                hipStream_t);
+                                float, int, int, int, int, int, int, int, int,
+                                int, float, hipStream_t);
 template <typename T>
 void launch_ssd_scan(float*, const T*, long, const T*, long, const float*,
                      const float*, const float*, float*, const int*, const int*,
@@ -238,8 +238,10 @@ void paged_attention_any(torch::Tensor out, torch::Tensor q, torch::Tensor k_cac
                          torch::Tensor v_cache, torch::Tensor block_tables,
                          c10::optional<torch::Tensor> query_start_loc,
                          torch::Tensor seq_lens, double scale,
-                         int64_t max_query_len) {
+                         int64_t max_query_len, int64_t window, bool has_sink,
+                         double sink) {
   TORCH_CHECK(q.is_cuda() && q.dim() == 3 && out.dim() == 3);
+  TORCH_CHECK(window >= 0, "window");
   const int rows = q.size(0), heads = q.size(1), dim = q.size(2);
   TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() &&
               k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.size(3) == dim &&
@@ -279,7 +281,7 @@ void paged_attention_any(torch::Tensor out, torch::Tensor q, torch::Tensor k_cac
         (long)q.stride(0), ptr<scalar_t>(k_cache), ptr<scalar_t>(v_cache),
         ptr<int>(block_tables), (int)block_tables.stride(0), qsl,
         ptr<int>(seq_lens), nseq, (float)scale, rows, heads, kv_heads, dim, vdim,
-        block_size, vec_ok, stream());
+        block_size, vec_ok, (int)window, has_sink ? 1 : 0, (float)sink, stream());
   });
 }
 

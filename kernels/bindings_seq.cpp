@@ -26,11 +26,11 @@ template <typename T>
 void launch_softcap(float*, const T*, float, long, hipStream_t);
 template <typename T>
 void launch_rope_partial(T*, long, long, const long*, const float*, int, int,
-                         int, int, hipStream_t);
+                         int, int, int, float, hipStream_t);
 template <typename T>
 void launch_latent_kv_write(const T*, const float*, float, const long*,
                             const float*, int, T*, const long*, int, int, int,
-                            hipStream_t);
+                            long, int, float, hipStream_t);
 template <typename T>
 void launch_causal_conv_state(T*, const T*, const float*, T*, const int*,
                               const int*, const int*, int, int, int, int, int,
@@ -38,6 +38,9 @@ void launch_causal_conv_state(T*, const T*, const float*, T*, const int*,
 // layer norms of the stream, attention of any shape, recurrences
 // (bindings_rec.cpp)
 void register_rec_ops(pybind11::module& m);
+// two-norm residual kernel, rotation + cache write, gates, squared relu,
+// expert router and combine (bindings_par.cpp)
+void register_par_ops(pybind11::module& m);
 namespace {
 
 hipStream_t stream() { return at::hip::getCurrentHIPStream().stream(); }
@@ -187,7 +190,8 @@ void softcap(torch::Tensor out, torch::Tensor in, double cap) {
 }
 
 void rope_partial(torch::Tensor x, torch::Tensor positions,
-                  torch::Tensor inv_freq, int64_t offset, int64_t rot_dims) {
+                  torch::Tensor inv_freq, int64_t offset, int64_t rot_dims,
+                  bool interleaved, double mag) {
   TORCH_CHECK(x.is_cuda() && x.dim() == 3 && x.stride(2) == 1);
   check_i64(positions, "positions");
   check_f32(inv_freq, "inv_freq");
@@ -200,15 +204,16 @@ void rope_partial(torch::Tensor x, torch::Tensor positions,
     launch_rope_partial<scalar_t>(ptr<scalar_t>(x), x.stride(0), x.stride(1),
                                   ptr<long>(positions), ptr<float>(inv_freq),
                                   (int)x.size(0), (int)x.size(1), (int)offset,
-                                  half, stream());
+                                  half, interleaved ? 1 : 0, (float)mag,
+                                  stream());
   });
 }
 
 void latent_kv_write(torch::Tensor dkv, torch::Tensor norm_w, double eps,
                      torch::Tensor positions, torch::Tensor inv_freq,
                      int64_t rot_dims, torch::Tensor cache,
-                     torch::Tensor slot_mapping) {
-  TORCH_CHECK(dkv.is_cuda() && dkv.is_contiguous() && dkv.dim() == 2);
+                     torch::Tensor slot_mapping, bool interleaved, double mag) {
+  TORCH_CHECK(dkv.is_cuda() && dkv.dim() == 2 && dkv.stride(1) == 1);
   check_f32(norm_w, "norm_w");
   check_f32(inv_freq, "inv_freq");
   check_i64(positions, "positions");
@@ -226,7 +231,8 @@ void latent_kv_write(torch::Tensor dkv, torch::Tensor norm_w, double eps,
     launch_latent_kv_write<scalar_t>(
         ptr<scalar_t>(dkv), ptr<float>(norm_w), (float)eps, ptr<long>(positions),
         ptr<float>(inv_freq), (int)(rot_dims / 2), ptr<scalar_t>(cache),
-        ptr<long>(slot_mapping), (int)dkv.size(0), rank, rot, stream());
+        ptr<long>(slot_mapping), (int)dkv.size(0), rank, rot,
+        (long)dkv.stride(0), interleaved ? 1 : 0, (float)mag, stream());
   });
 }
 
@@ -278,4 +284,5 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("latent_kv_write", &latent_kv_write);
   m.def("causal_conv_state", &causal_conv_state);
   register_rec_ops(m);
+  register_par_ops(m);
 }

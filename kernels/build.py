@@ -14,8 +14,9 @@ Several extensions, so that a model only builds the ones it uses
             and MFMA) + bindings_attn.cpp, module_attn.cpp
 ``_C_seq``  f32-residual-stream ops (RMS and layer norms), short causal
             convolution with per-sequence state, grouped-query attention of
-            any shape, recurrences with per-sequence state + bindings_seq.cpp,
-            bindings_rec.cpp
+            any shape, recurrences with per-sequence state, two-norm blocks,
+            rotation + cache write, gates, expert routing, the grouped expert
+            product + bindings_seq.cpp, bindings_rec.cpp, bindings_par.cpp
 ``_C_lat``  windowed latent attention with sinks + bindings_lat.cpp
 """
 
@@ -34,7 +35,9 @@ PKG = REPO / "vllm_tgis_adapter_amd"
 ARCH = os.environ.get("PYTORCH_ROCM_ARCH", "gfx950")
 
 _SEQ_SOURCES = ["stream_ops.hip", "canon_conv.hip", "layer_norm_stream.hip",
-                "paged_attention_any.hip", "recurrent_scan.hip"]
+                "paged_attention_any.hip", "recurrent_scan.hip", "gated_block.hip"]
+# kernels without torch types that more than one extension links
+_SHARED_SOURCES = ["moe_gemm.hip"]
 _LAT_SOURCES = ["latent_attention.hip", "latent_attention_mfma.hip"]
 _ATTN_SOURCES = ["attention.hip", "attention_decode_mfma.hip",
                  "attention_prefill_mfma.hip", "attention_prefill_mfma_v2.hip"]
@@ -50,8 +53,9 @@ EXTENSIONS = {
         + [KERNELS / "bindings_attn.cpp", KERNELS / "module_attn.cpp"],
     ),
     "_C_seq": dict(
-        sources=lambda: [KERNELS / n for n in _SEQ_SOURCES]
-        + [KERNELS / "bindings_seq.cpp", KERNELS / "bindings_rec.cpp"],
+        sources=lambda: [KERNELS / n for n in _SEQ_SOURCES + _SHARED_SOURCES]
+        + [KERNELS / "bindings_seq.cpp", KERNELS / "bindings_rec.cpp",
+           KERNELS / "bindings_par.cpp"],
     ),
     "_C_lat": dict(
         sources=lambda: [KERNELS / n for n in _LAT_SOURCES] + [KERNELS / "bindings_lat.cpp"],

@@ -5,6 +5,7 @@
 //
 //   h[r, :]  = silu(x[r]·Wg_e^T) * (x[r]·Wu_e^T)   (gated, w13 = [E, 2I, H])
 //   y[r, :]  = h[r]·W2_e^T                          (plain, w2  = [E, H, I])
+//   a[r, :]  = relu(x[r]·Wu_e^T)^2                  (squared relu, w = [E, I, H])
 // where e = the expert owning sorted row r (seg_off[e] <= r < seg_off[e+1]).
 //
 // Geometry per kernel: grid (N/128, E * MBLK); each workgroup owns one
@@ -26,7 +27,8 @@ DEVINLINE int mg_swz(int row, int byte_in_row) {
   return row * (MG_KB * 2) + (byte_in_row ^ ((row & 7) << 4));
 }
 
-template <bool GATED>
+// MODE 0: plain, 1: gated (silu(g) * u), 2: squared relu
+template <int MODE>
 __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(
     __hip_bfloat16* __restrict__ y,        // [T, N_out] (N_out = I or H)
     const __hip_bfloat16* __restrict__ x,  // [T, K] sorted by expert
@@ -36,6 +38,7 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(
     const int N,   // output width (I for gated, H for plain)
     const int K,
     const int MBLK) {
+  constexpr bool GATED = MODE == 1;
   const int n_blk = blockIdx.x;
   const int e = blockIdx.y / MBLK;
   const int mb = blockIdx.y % MBLK;
@@ -159,6 +162,9 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(
         if (GATED) {
           const float act = v / (1.f + __expf(-v));
           v = act * acc_u[mt][nt][r];
+        } else if (MODE == 2) {
+          v = fmaxf(v, 0.f);
+          v = v * v;
         }
         y[(long)(m_lo + m) * N + n] = __float2bfloat16(v);
       }
@@ -168,14 +174,17 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(
 
 void launch_moe_gemm(__hip_bfloat16* y, const __hip_bfloat16* x,
                      const __hip_bfloat16* w, const int* seg_off, int E,
-                     int N, int K, int T, bool gated, hipStream_t stream) {
+                     int N, int K, int T, int mode, hipStream_t stream) {
   const int mblk = (T + 127) / 128;
   dim3 grid(N / 128, E * mblk);
   dim3 block(256);
-  if (gated)
-    hipLaunchKernelGGL(moe_gemm_kernel<true>, grid, block, 0, stream, y, x, w,
+  if (mode == 1)
+    hipLaunchKernelGGL(moe_gemm_kernel<1>, grid, block, 0, stream, y, x, w,
+                       seg_off, E, N, K, mblk);
+  else if (mode == 2)
+    hipLaunchKernelGGL(moe_gemm_kernel<2>, grid, block, 0, stream, y, x, w,
                        seg_off, E, N, K, mblk);
   else
-    hipLaunchKernelGGL(moe_gemm_kernel<false>, grid, block, 0, stream, y, x,
-                       w, seg_off, E, N, K, mblk);
+    hipLaunchKernelGGL(moe_gemm_kernel<0>, grid, block, 0, stream, y, x, w,
+                       seg_off, E, N, K, mblk);
 }

@@ -5,8 +5,10 @@
 //   k_cache [blocks, block, G, dim]     v_cache [blocks, block, G, vdim]
 //   q [rows, H, dim]  ->  out [rows, H, vdim]
 //
-// Query head h reads key/value head h / (H / G).  One workgroup per (query
-// row, head).  Per tile of 256 keys:
+// Query head h reads key/value head h / (H / G).  A query at position i sees
+// keys j with 0 <= i - j < window (window 0: every j <= i); with a sink the
+// softmax denominator also holds exp(sink), a key without a value.  One
+// workgroup per (query row, head).  Per tile of 256 keys:
 //   phase 1  thread j scores key j (q, already multiplied by the score scale,
 //            broadcast from LDS; the key row read with 16-byte loads), block
 //            max / sum give the online-softmax step
@@ -58,7 +60,8 @@ __global__ __launch_bounds__(PA_THREADS) void paged_attention_any_kernel(
     const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ qsl, const int* __restrict__ seq_lens, int nseq,
     float scale, int heads, int kv_heads, int dim, int vdim, int block_size,
-    int vp /* pow2 >= min(vdim, 256) */, int vec_ok) {
+    int vp /* pow2 >= min(vdim, 256) */, int vec_ok, int window, int has_sink,
+    float sink) {
   extern __shared__ float smem[];
   float* q_s = smem;                               // [dim]
   float* p_s = q_s + ((dim + 1) & ~1);             // [256]
@@ -107,7 +110,8 @@ __global__ __launch_bounds__(PA_THREADS) void paged_attention_any_kernel(
   for (int i = 0; i < PA_MAX_DPT; ++i) acc[i] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
 
-  for (int base = 0; base < ctx; base += PA_THREADS) {
+  const int first = (window > 0 && ctx > window) ? ctx - window : 0;
+  for (int base = first; base < ctx; base += PA_THREADS) {
     const int j = base + tid;
     float s = -INFINITY;
     if (j < ctx) {
@@ -149,7 +153,12 @@ __global__ __launch_bounds__(PA_THREADS) void paged_attention_any_kernel(
     __syncthreads();   // p_s / tok_s are rewritten by the next tile
   }
 
-  const float inv = 1.0f / l_run;
+  float inv = 1.0f / l_run;
+  if (has_sink) {
+    const float m_fin = fmaxf(m_run, sink);
+    const float rescale = expf(m_run - m_fin);
+    inv = rescale / (l_run * rescale + expf(sink - m_fin));
+  }
   if (groups > 1) {
     // vdim <= vp <= 128 here: one dim per thread, sum the groups through LDS
     acc_s[tid] = acc[0];
@@ -177,6 +186,7 @@ void launch_paged_attention_any(T* out, long o_st, const T* q, long q_st,
                                 const int* qsl, const int* seq_lens, int nseq,
                                 float scale, int rows, int heads, int kv_heads,
                                 int dim, int vdim, int block_size, int vec_ok,
+                                int window, int has_sink, float sink,
                                 hipStream_t stream) {
   int vp = 1;
   while (vp < vdim && vp < PA_THREADS) vp <<= 1;
@@ -185,14 +195,15 @@ void launch_paged_attention_any(T* out, long o_st, const T* q, long q_st,
   dim3 grid(rows, heads);
   paged_attention_any_kernel<T><<<grid, PA_THREADS, smem, stream>>>(
       out, o_st, q, q_st, k_cache, v_cache, block_tables, bt_stride, qsl,
-      seq_lens, nseq, scale, heads, kv_heads, dim, vdim, block_size, vp, vec_ok);
+      seq_lens, nseq, scale, heads, kv_heads, dim, vdim, block_size, vp, vec_ok,
+      window, has_sink, sink);
 }
 
 template void launch_paged_attention_any<float>(
     float*, long, const float*, long, const float*, const float*, const int*, int,
-    const int*, const int*, int, float, int, int, int, int, int, int, int,
-    hipStream_t);
+    const int*, const int*, int, float, int, int, int, int, int, int, int, int,
+    int, float, hipStream_t);
 template void launch_paged_attention_any<__hip_bfloat16>(
     __hip_bfloat16*, long, const __hip_bfloat16*, long, const __hip_bfloat16*,
     const __hip_bfloat16*, const int*, int, const int*, const int*, int, float,
-    int, int, int, int, int, int, int, hipStream_t);
+    int, int, int, int, int, int, int, int, int, float, hipStream_t);

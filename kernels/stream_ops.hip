@@ -225,13 +225,16 @@ __global__ void softcap_kernel(float* __restrict__ out, const T* __restrict__ in
     out[i] = cap * tanhf(ScalarOps<T>::to_f32(in[i]) * inv);
 }
 
-// Half-split rotation of dims [offset, offset + 2*half) of every head of
-// x [T, H, D] (strided), in place.  Angle = float(position) * inv_freq[i].
+// Rotation of dims [offset, offset + 2*half) of every head of x [T, H, D]
+// (strided), in place: pair i is dims (i, i + half), or (2i, 2i + 1) when
+// `interleaved`.  Angle = float(position) * inv_freq[i]; cos and sin are
+// multiplied by `mag`.
 template <typename T>
 __global__ void rope_partial_kernel(T* __restrict__ x, long st, long sh,
                                     const long* __restrict__ positions,
                                     const float* __restrict__ inv_freq,
-                                    int heads, int offset, int half, long n) {
+                                    int heads, int offset, int half, long n,
+                                    int interleaved, float mag) {
   for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n;
        i += (long)gridDim.x * blockDim.x) {
     const int k = (int)(i % half);
@@ -241,17 +244,22 @@ __global__ void rope_partial_kernel(T* __restrict__ x, long st, long sh,
     const float ang = (float)positions[t] * inv_freq[k];
     float s, c;
     sincosf(ang, &s, &c);
+    s *= mag;
+    c *= mag;
     T* p = x + t * st + h * sh + offset;
-    const float u = ScalarOps<T>::to_f32(p[k]);
-    const float v = ScalarOps<T>::to_f32(p[k + half]);
-    p[k] = ScalarOps<T>::from_f32(u * c - v * s);
-    p[k + half] = ScalarOps<T>::from_f32(v * c + u * s);
+    const int ia = interleaved ? 2 * k : k;
+    const int ib = interleaved ? 2 * k + 1 : k + half;
+    const float u = ScalarOps<T>::to_f32(p[ia]);
+    const float v = ScalarOps<T>::to_f32(p[ib]);
+    p[ia] = ScalarOps<T>::from_f32(u * c - v * s);
+    p[ib] = ScalarOps<T>::from_f32(v * c + u * s);
   }
 }
 
 // One workgroup per token: RMS-norm the first `rank` values of the row with a
-// plain weight, rotate the first 2*half of the remaining `rot` values, store
-// the row at its slot of the paged cache (slot < 0: padding row, skipped).
+// plain weight, rotate the first 2*half of the remaining `rot` values (pairs
+// and `mag` as in rope_partial), store the row at its slot of the paged cache
+// (slot < 0: padding row, skipped).  Input rows are `in_st` elements apart.
 template <typename T>
 __global__ void latent_kv_write_kernel(const T* __restrict__ dkv,
                                        const float* __restrict__ norm_w,
@@ -260,12 +268,13 @@ __global__ void latent_kv_write_kernel(const T* __restrict__ dkv,
                                        const float* __restrict__ inv_freq,
                                        int half, T* __restrict__ cache,
                                        const long* __restrict__ slot_mapping,
-                                       int rank, int rot) {
+                                       int rank, int rot, long in_st,
+                                       int interleaved, float mag) {
   const long t = blockIdx.x;
   const long slot = slot_mapping[t];
   if (slot < 0) return;
   const int d = rank + rot;
-  const T* in = dkv + t * d;
+  const T* in = dkv + t * in_st;
   T* out = cache + slot * d;
   float ss = 0.f;
   for (int c = threadIdx.x; c < rank; c += blockDim.x) {
@@ -281,10 +290,14 @@ __global__ void latent_kv_write_kernel(const T* __restrict__ dkv,
   for (int k = threadIdx.x; k < half; k += blockDim.x) {
     float s, c;
     sincosf(pos * inv_freq[k], &s, &c);
-    const float u = ScalarOps<T>::to_f32(in[rank + k]);
-    const float v = ScalarOps<T>::to_f32(in[rank + k + half]);
-    out[rank + k] = ScalarOps<T>::from_f32(u * c - v * s);
-    out[rank + k + half] = ScalarOps<T>::from_f32(v * c + u * s);
+    s *= mag;
+    c *= mag;
+    const int ia = rank + (interleaved ? 2 * k : k);
+    const int ib = rank + (interleaved ? 2 * k + 1 : k + half);
+    const float u = ScalarOps<T>::to_f32(in[ia]);
+    const float v = ScalarOps<T>::to_f32(in[ib]);
+    out[ia] = ScalarOps<T>::from_f32(u * c - v * s);
+    out[ib] = ScalarOps<T>::from_f32(v * c + u * s);
   }
   for (int k = 2 * half + threadIdx.x; k < rot; k += blockDim.x)
     out[rank + k] = in[rank + k];
@@ -357,18 +370,20 @@ void launch_softcap(float* out, const T* in, float cap, long n, hipStream_t s) {
 template <typename T>
 void launch_rope_partial(T* x, long st, long sh, const long* positions,
                          const float* inv_freq, int rows, int heads, int offset,
-                         int half, hipStream_t s) {
+                         int half, int interleaved, float mag, hipStream_t s) {
   const long n = (long)rows * heads * half;
   rope_partial_kernel<T><<<grid_for(n, 256), 256, 0, s>>>(
-      x, st, sh, positions, inv_freq, heads, offset, half, n);
+      x, st, sh, positions, inv_freq, heads, offset, half, n, interleaved, mag);
 }
 template <typename T>
 void launch_latent_kv_write(const T* dkv, const float* norm_w, float eps,
                             const long* positions, const float* inv_freq,
                             int half, T* cache, const long* slot_mapping,
-                            int rows, int rank, int rot, hipStream_t s) {
+                            int rows, int rank, int rot, long in_st,
+                            int interleaved, float mag, hipStream_t s) {
   latent_kv_write_kernel<T><<<rows, 128, 0, s>>>(
-      dkv, norm_w, eps, positions, inv_freq, half, cache, slot_mapping, rank, rot);
+      dkv, norm_w, eps, positions, inv_freq, half, cache, slot_mapping, rank, rot,
+      in_st, interleaved, mag);
 }
 
 #define INSTANTIATE(T)                                                          \
@@ -386,11 +401,11 @@ void launch_latent_kv_write(const T* dkv, const float* norm_w, float eps,
                                               hipStream_t);                     \
   template void launch_softcap<T>(float*, const T*, float, long, hipStream_t);  \
   template void launch_rope_partial<T>(T*, long, long, const long*,             \
-                                       const float*, int, int, int, int,        \
-                                       hipStream_t);                            \
+                                       const float*, int, int, int, int, int,   \
+                                       float, hipStream_t);                     \
   template void launch_latent_kv_write<T>(const T*, const float*, float,        \
                                           const long*, const float*, int, T*,   \
-                                          const long*, int, int, int,           \
-                                          hipStream_t);
+                                          const long*, int, int, int, long,     \
+                                          int, float, hipStream_t);
 INSTANTIATE(float)
 INSTANTIATE(__hip_bfloat16)
