@@ -45,7 +45,7 @@ def parse_args():
     p.add_argument("--arch-sizes", type=str, default="s,m",
                    help="arch mode: comma list of sizes (s, m)")
     p.add_argument("--arch-models", type=str, default="dolodra,llama",
-                   help="arch mode: which models to run (dolodra, kezunex, llama)")
+                   help="arch mode: which models to run (dolodra, kezunex, relerax, llama)")
     p.add_argument("--model", type=str, default="llama-3-8b")
     p.add_argument("--batch", type=int, default=512)
     p.add_argument("--prompt-len", type=int, default=512)
@@ -562,6 +562,46 @@ def _kezunex_model_config(name: str, sz: dict, dtype: str):
     return mc
 
 
+# Relerax at the same widths: eight two-norm parallel layers, latent attention
+# (the latent sizes of the Dolodra config above, no window) in three of four
+# layers and windowed grouped-query attention with a sink (the llama's head
+# shape) in the fourth; dense squared-relu feed-forwards alternate with routed
+# ones whose chosen experts add up to about the dense size.
+RELERAX_SIZES = {
+    "s": dict(experts=16, identity=4, top=4, expert_ff=2048),
+    "m": dict(experts=16, identity=4, top=4, expert_ff=5376),
+    "t": dict(experts=4, identity=2, top=2, expert_ff=96),
+}
+
+
+def _relerax_model_config(name: str, sz: dict, dtype: str):
+    from vllm_tgis_adapter_amd.engine.config import _DTYPES
+    from vllm_tgis_adapter_amd.models.relerax import model_config_from_json
+
+    rx = RELERAX_SIZES[name]
+    scaling = {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}
+    latent = {"heads": sz["heads"], "dim": sz["dim"], "rot_dim": sz["rot"], "vdim": sz["vdim"],
+              "kv_rank": sz["rank"], "scale": (sz["dim"] + sz["rot"]) ** -0.5,
+              "rot": {"base": 10000.0, "dims": sz["rot"], "scaling": scaling}}
+    hd = sz["width"] // sz["heads"]
+    attn = {"heads": sz["heads"], "kv_heads": sz["llama_kv_heads"], "dim": hd, "vdim": hd,
+            "scale": hd ** -0.5, "mask": {"size": sz["window"]},
+            "rot": {"base": 10000.0, "dims": hd // 2, "scaling": scaling}}
+    dense = {"kind": "dense", "ff": sz["ff"]}
+    moe = {"kind": "moe", "expert": {"ff": rx["expert_ff"]},
+           "router": {"experts": rx["experts"], "identity": rx["identity"], "top": rx["top"]}}
+    layers = []
+    for i in range(sz["layers"]):
+        kind = "attention" if i % 4 == 2 else "latent_attention"
+        layers.append({"type": kind, "mixer": attn if kind == "attention" else latent,
+                       "mlp": moe if i % 2 == 1 else dense})
+    hf = {"architecture": "Relerax", "vocab": sz["vocab"], "width": sz["width"],
+          "layers": layers, "norm": {"eps": 1e-5}}
+    mc = model_config_from_json("relerax-synthetic", hf)
+    mc.dtype = _DTYPES[dtype]
+    return mc
+
+
 def _arch_measure(mc, args, device: str, batch: int, prompt_len: int, steps: int,
                   warmup: int) -> dict:
     from vllm_tgis_adapter_amd.engine import EngineConfig, LLMEngine, SamplingParams
@@ -622,12 +662,14 @@ def run_arch(args, device: str) -> None:
         plen = args.prompt_len if device == "cuda" else 32
         steps = args.steps if device == "cuda" else 4
         warm = args.warmup if device == "cuda" else 1
-        models = [("dolodra", dolo), ("kezunex", None), ("llama", llama)]
+        models = [("dolodra", dolo), ("kezunex", None), ("relerax", None), ("llama", llama)]
         for label, mc in models:
             if label not in args.arch_models.split(","):
                 continue
             if label == "kezunex":
                 mc = _kezunex_model_config(name, sz, args.dtype)
+            if label == "relerax":
+                mc = _relerax_model_config(name, sz, args.dtype)
             r = _arch_measure(mc, args, device, batch, plen, steps, warm)
             r.update(size=name, model=label, batch=batch, prompt_len=plen)
             out.append(r)

@@ -41,7 +41,11 @@ DEVINLINE bf16x8_t load_kv8<unsigned char>(const unsigned char* p) {
 #define KVT 32     // kv slots per mfma tile
 #define NWAVES 4   // waves per workgroup
 
-template <int HEAD_DIM, typename CT>
+// WS (window + sink variant): the query (position seq_len - 1) sees the last
+// `window` keys only (window 0: all), and the probabilities enter the value
+// product as the sum of two bf16 terms (rounded value + rounded remainder);
+// the sink joins the denominator in the merge kernel.
+template <int HEAD_DIM, typename CT, bool WS>
 __global__ __launch_bounds__(256, 2) void paged_decode_mfma_kernel(
     float* __restrict__ part_acc,   // [nseq, nheads, P, HEAD_DIM] f32
     float* __restrict__ part_ml,    // [nseq, nheads, P, 2] f32 (m, l)
@@ -55,7 +59,8 @@ __global__ __launch_bounds__(256, 2) void paged_decode_mfma_kernel(
     const int kvh,
     const int group,       // nheads / kvh, <= 8
     const int block_size,
-    const int max_blocks) {
+    const int max_blocks,
+    const int window) {
   constexpr int KCH = HEAD_DIM / 16;  // k-chunks for the QK^T mfma
   constexpr int DT = HEAD_DIM / 32;   // 32-col output tiles
 
@@ -73,8 +78,10 @@ __global__ __launch_bounds__(256, 2) void paged_decode_mfma_kernel(
 
   // this partition's tile range; waves stride by NWAVES inside it
   const int tiles_total = (seq_len + KVT - 1) / KVT;
-  const int tpp = (tiles_total + npart - 1) / npart;
-  const int tile_lo = part * tpp;
+  const int first_pos = (WS && window > 0) ? max(0, seq_len - window) : 0;
+  const int tile_first = first_pos / KVT;
+  const int tpp = (tiles_total - tile_first + npart - 1) / npart;
+  const int tile_lo = tile_first + part * tpp;
   const int tile_hi = min(tile_lo + tpp, tiles_total);
 
   const int head0 = kv_head * group;
@@ -169,7 +176,7 @@ __global__ __launch_bounds__(256, 2) void paged_decode_mfma_kernel(
     for (int r = 0; r < 16; ++r) {
       const int kv_pos = kv_base + (r & 3) + 8 * (r >> 2) + 4 * half;
       float sv = acc_s[r] * scale;
-      if (kv_pos >= seq_len) sv = -FLT_MAX;
+      if (kv_pos >= seq_len || (WS && kv_pos < first_pos)) sv = -FLT_MAX;
       s_val[r] = sv;
       local_max = fmaxf(local_max, sv);
     }
@@ -201,26 +208,34 @@ __global__ __launch_bounds__(256, 2) void paged_decode_mfma_kernel(
     }
 
     // ---- pack P to bf16 A-fragments (cvt_pk + permlane32_swap) -----------
-    unsigned int pk[8];
+    constexpr int PASSES = WS ? 2 : 1;   // pass 1: what the first rounding left over
+    bf16x8_t pa[PASSES][2];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2"
-                   : "=v"(pk[i]) : "v"(p[2 * i]), "v"(p[2 * i + 1]));
-    }
-    bf16x8_t pa[2];
+    for (int ps = 0; ps < PASSES; ++ps) {
+      unsigned int pk[8];
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      unsigned x0 = pk[4 * c + 0], x1 = pk[4 * c + 1];
-      unsigned y0 = pk[4 * c + 2], y1 = pk[4 * c + 3];
-      {
-        auto r0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
-        x0 = r0[0]; y0 = r0[1];
-        auto r1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
-        x1 = r1[0]; y1 = r1[1];
+      for (int i = 0; i < 8; ++i) {
+        asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2"
+                     : "=v"(pk[i]) : "v"(p[2 * i]), "v"(p[2 * i + 1]));
+        if (WS && ps == 0) {
+          p[2 * i] -= __uint_as_float(pk[i] << 16);
+          p[2 * i + 1] -= __uint_as_float(pk[i] & 0xffff0000u);
+        }
       }
-      union { unsigned u[4]; bf16x8_t v; } u;
-      u.u[0] = x0; u.u[1] = x1; u.u[2] = y0; u.u[3] = y1;
-      pa[c] = u.v;
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        unsigned x0 = pk[4 * c + 0], x1 = pk[4 * c + 1];
+        unsigned y0 = pk[4 * c + 2], y1 = pk[4 * c + 3];
+        {
+          auto r0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+          x0 = r0[0]; y0 = r0[1];
+          auto r1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+          x1 = r1[0]; y1 = r1[1];
+        }
+        union { unsigned u[4]; bf16x8_t v; } u;
+        u.u[0] = x0; u.u[1] = x1; u.u[2] = y0; u.u[3] = y1;
+        pa[ps][c] = u.v;
+      }
     }
 
     // ---- PV: out[q][d] += P[q][kv] V[kv][d] ------------------------------
@@ -233,7 +248,10 @@ __global__ __launch_bounds__(256, 2) void paged_decode_mfma_kernel(
         for (int j = 0; j < 8; ++j)
           b[j] = *reinterpret_cast<const short*>(
               v_lds + (c * 16 + half * 8 + j) * HEAD_DIM + dt * 32 + col);
-        acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pa[c], b, acc_o[dt], 0, 0, 0);
+        acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pa[0][c], b, acc_o[dt], 0, 0, 0);
+        if (WS)
+          acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pa[PASSES - 1][c], b,
+                                                              acc_o[dt], 0, 0, 0);
       }
     }
   }
@@ -264,7 +282,9 @@ __global__ void decode_merge_kernel(
     const float* __restrict__ part_acc,    // [nseq, nheads, P, HD]
     const float* __restrict__ part_ml,     // [nseq, nheads, P, 2]
     const int nheads,
-    const int P) {
+    const int P,
+    const int has_sink,
+    const float sink) {
   const int seq = blockIdx.x;
   const int head = blockIdx.y;
   const int d = threadIdx.x;
@@ -275,6 +295,10 @@ __global__ void decode_merge_kernel(
   float M = -FLT_MAX;
   for (int p = 0; p < P; ++p) M = fmaxf(M, ml[2 * p]);
   float L = 0.f, A = 0.f;
+  if (has_sink) {   // a key without a value: only the denominator sees it
+    M = fmaxf(M, sink);
+    L = __expf(sink - M);
+  }
   for (int p = 0; p < P; ++p) {
     const float f = __expf(ml[2 * p] - M);
     L += f * ml[2 * p + 1];
@@ -302,26 +326,49 @@ static void launch_decode_ct(__hip_bfloat16* out, float* part_acc,
                              const CT* kc, const CT* vc, const int* bt,
                              const int* sl, float scale, int nseq, int nheads,
                              int kvh, int head_dim, int block_size,
-                             int max_blocks, int npart, hipStream_t stream) {
+                             int max_blocks, int npart, hipStream_t stream,
+                             int window = 0, int has_sink = 0, float sink = 0.f,
+                             bool ws = false) {
   const int group = nheads / kvh;
   dim3 grid(nseq, kvh, npart);
   dim3 block(256);
   dim3 mgrid(nseq, nheads);
   const int P = npart * NWAVES;
+  if (ws) {
+    switch (head_dim) {
+      case 64:
+        hipLaunchKernelGGL((paged_decode_mfma_kernel<64, CT, true>), grid, block, 0,
+                           stream, part_acc, part_ml, q, kc, vc, bt, sl, scale,
+                           nheads, kvh, group, block_size, max_blocks, window);
+        hipLaunchKernelGGL(decode_merge_kernel<64>, mgrid, dim3(64), 0, stream,
+                           out, part_acc, part_ml, nheads, P, has_sink, sink);
+        break;
+      case 128:
+        hipLaunchKernelGGL((paged_decode_mfma_kernel<128, CT, true>), grid, block, 0,
+                           stream, part_acc, part_ml, q, kc, vc, bt, sl, scale,
+                           nheads, kvh, group, block_size, max_blocks, window);
+        hipLaunchKernelGGL(decode_merge_kernel<128>, mgrid, dim3(128), 0, stream,
+                           out, part_acc, part_ml, nheads, P, has_sink, sink);
+        break;
+      default:
+        abort();
+    }
+    return;
+  }
   switch (head_dim) {
     case 64:
-      hipLaunchKernelGGL((paged_decode_mfma_kernel<64, CT>), grid, block, 0,
+      hipLaunchKernelGGL((paged_decode_mfma_kernel<64, CT, false>), grid, block, 0,
                          stream, part_acc, part_ml, q, kc, vc, bt, sl, scale,
-                         nheads, kvh, group, block_size, max_blocks);
+                         nheads, kvh, group, block_size, max_blocks, 0);
       hipLaunchKernelGGL(decode_merge_kernel<64>, mgrid, dim3(64), 0, stream,
-                         out, part_acc, part_ml, nheads, P);
+                         out, part_acc, part_ml, nheads, P, 0, 0.f);
       break;
     case 128:
-      hipLaunchKernelGGL((paged_decode_mfma_kernel<128, CT>), grid, block, 0,
+      hipLaunchKernelGGL((paged_decode_mfma_kernel<128, CT, false>), grid, block, 0,
                          stream, part_acc, part_ml, q, kc, vc, bt, sl, scale,
-                         nheads, kvh, group, block_size, max_blocks);
+                         nheads, kvh, group, block_size, max_blocks, 0);
       hipLaunchKernelGGL(decode_merge_kernel<128>, mgrid, dim3(128), 0, stream,
-                         out, part_acc, part_ml, nheads, P);
+                         out, part_acc, part_ml, nheads, P, 0, 0.f);
       break;
     default:
       abort();
@@ -349,4 +396,19 @@ void launch_paged_decode_mfma_fp8(
   launch_decode_ct<unsigned char>(out, part_acc, part_ml, q, kc, vc, bt, sl,
                                   scale, nseq, nheads, kvh, head_dim,
                                   block_size, max_blocks, npart, stream);
+}
+
+// window + sink variant (bf16 cache)
+void launch_paged_decode_mfma_ws(__hip_bfloat16* out, float* part_acc,
+                                 float* part_ml, const __hip_bfloat16* q,
+                                 const __hip_bfloat16* kc, const __hip_bfloat16* vc,
+                                 const int* bt, const int* sl, float scale,
+                                 int nseq, int nheads, int kvh, int head_dim,
+                                 int block_size, int max_blocks, int npart,
+                                 int window, int has_sink, float sink,
+                                 hipStream_t stream) {
+  launch_decode_ct<__hip_bfloat16>(out, part_acc, part_ml, q, kc, vc, bt, sl,
+                                   scale, nseq, nheads, kvh, head_dim,
+                                   block_size, max_blocks, npart, stream, window,
+                                   has_sink, sink, true);
 }

@@ -58,7 +58,12 @@ __device__ inline float cross_half_sum(float v) {
   return v + __shfl_xor(v, 32, 64);
 }
 
-template <int HEAD_DIM, typename CT, int NW>
+// WS (window + sink variant): a query at position i sees keys j with
+// 0 <= i - j < window (window 0: all j <= i); with has_sink the denominator
+// also holds exp(sink); and the probabilities enter the value product as the
+// sum of two bf16 terms (rounded value + rounded remainder), so that they
+// carry 16 mantissa bits instead of 8.
+template <int HEAD_DIM, typename CT, int NW, bool WS>
 __global__ __launch_bounds__(NW * 64, 512 / (NW * 64)) void paged_prefill_mfma_v2_kernel(
     __hip_bfloat16* __restrict__ out,            // [total_q, nheads, HD]
     const __hip_bfloat16* __restrict__ q,        // [total_q, nheads, HD]
@@ -71,7 +76,10 @@ __global__ __launch_bounds__(NW * 64, 512 / (NW * 64)) void paged_prefill_mfma_v
     const int nheads,
     const int kvh,
     const int block_size,
-    const int max_blocks) {
+    const int max_blocks,
+    const int window,
+    const int has_sink,
+    const float sink) {
   static_assert(HEAD_DIM == 128, "v2 is specialised for HD=128");
   constexpr int KCH = HEAD_DIM / 16;  // QK^T k-chunks (8)
   constexpr int DT = HEAD_DIM / 32;   // 32-col output tiles (4)
@@ -134,6 +142,13 @@ __global__ __launch_bounds__(NW * 64, 512 / (NW * 64)) void paged_prefill_mfma_v
   const int wave_max_pos =
       seq_len - q_len + tile_base + wave * 32 + max(wave_rows - 1, 0);
   const int wave_q_pos_min = seq_len - q_len + tile_base + wave * 32;
+  // first key tile any row of the workgroup sees, lowest key position any
+  // row of this wave sees
+  int kv_first = 0, wave_win_lo = 0;
+  if (WS && window > 0) {
+    kv_first = max(0, seq_len - q_len + tile_base - window + 1) / KVT2 * KVT2;
+    wave_win_lo = max(0, wave_q_pos_min - window + 1);
+  }
 
   // ---- staging map: thread t covers slot (t % ROWS_PER_PASS, t / RPP * 8)
   // with ROWS_PER_PASS = NTHREADS/16 rows per pass (16 8-elem slots per row)
@@ -171,19 +186,20 @@ __global__ __launch_bounds__(NW * 64, 512 / (NW * 64)) void paged_prefill_mfma_v
     }
   };
 
-  stage_load(0);
-  stage_write(0);
+  stage_load(kv_first);
+  stage_write((kv_first / KVT2) & 1);
 
   const float sc2 = scale * LOG2E;  // fold softmax scale into exp2 domain
 
-  for (int kv_base = 0; kv_base < kv_limit; kv_base += KVT2) {
+  for (int kv_base = kv_first; kv_base < kv_limit; kv_base += KVT2) {
     const int buf = (kv_base / KVT2) & 1;
     __syncthreads();  // publish tile (kv_base) to all waves
 
     // wave-uniform: MFMAs must run with a full EXEC mask — a per-lane guard
     // here drops the masked lanes' K fragments from the score MFMA
     const bool wave_active =
-        (tile_base + wave * 32 < q_len) && (kv_base <= wave_max_pos);
+        (tile_base + wave * 32 < q_len) && (kv_base <= wave_max_pos) &&
+        (!WS || kv_base + KVT2 > wave_win_lo);
     const char* k_lds = reinterpret_cast<const char*>(k_lds2[buf]);
     const char* v_lds = v_lds2[buf];
 
@@ -216,7 +232,9 @@ __global__ __launch_bounds__(NW * 64, 512 / (NW * 64)) void paged_prefill_mfma_v
       // fast path: tile strictly below every row's causal diagonal
       const bool full_tile = (kv_base + KVT2 - 1 <= wave_q_pos_min) &&
                              (kv_base + KVT2 <= seq_len) &&
-                             (tile_base + wave * 32 + 31 < q_len);
+                             (tile_base + wave * 32 + 31 < q_len) &&
+                             (!WS || window == 0 ||
+                              kv_base > wave_q_pos_min + 31 - window);
       float local_max = -FLT_MAX;
       if (full_tile) {
 #pragma unroll
@@ -232,7 +250,9 @@ __global__ __launch_bounds__(NW * 64, 512 / (NW * 64)) void paged_prefill_mfma_v
             const int kv_pos =
                 kv_base + kb * 32 + (r & 3) + 8 * (r >> 2) + 4 * half;
             float v = acc_s[kb][r];
-            if (!q_valid || kv_pos > q_pos || kv_pos >= seq_len) v = -FLT_MAX;
+            if (!q_valid || kv_pos > q_pos || kv_pos >= seq_len ||
+                (WS && window > 0 && kv_pos + window <= q_pos))
+              v = -FLT_MAX;
             acc_s[kb][r] = v;
             local_max = fmaxf(local_max, v);
           }
@@ -280,29 +300,38 @@ __global__ __launch_bounds__(NW * 64, 512 / (NW * 64)) void paged_prefill_mfma_v
       l_state += cross_half_sum(local_sum);
 
       // ---- P -> bf16 A-fragments (cvt_pk + permlane32_swap, T12) -------
-      bf16x8_t pa[4];
+      // PASSES 2 (WS): pass 1 packs what the first rounding left over
+      constexpr int PASSES = WS ? 2 : 1;
+      bf16x8_t pa[PASSES][4];
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        unsigned int pk[8];
+      for (int ps = 0; ps < PASSES; ++ps) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2"
-                       : "=v"(pk[i])
-                       : "v"(p[kb * 16 + 2 * i]), "v"(p[kb * 16 + 2 * i + 1]));
-        }
+        for (int kb = 0; kb < 2; ++kb) {
+          unsigned int pk[8];
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
-          unsigned x0 = pk[4 * c + 0], x1 = pk[4 * c + 1];
-          unsigned y0 = pk[4 * c + 2], y1 = pk[4 * c + 3];
-          {
-            auto r0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
-            x0 = r0[0]; y0 = r0[1];
-            auto r1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
-            x1 = r1[0]; y1 = r1[1];
+          for (int i = 0; i < 8; ++i) {
+            asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2"
+                         : "=v"(pk[i])
+                         : "v"(p[kb * 16 + 2 * i]), "v"(p[kb * 16 + 2 * i + 1]));
+            if (WS && ps == 0) {
+              p[kb * 16 + 2 * i] -= __uint_as_float(pk[i] << 16);
+              p[kb * 16 + 2 * i + 1] -= __uint_as_float(pk[i] & 0xffff0000u);
+            }
           }
-          union { unsigned u[4]; bf16x8_t v; } u;
-          u.u[0] = x0; u.u[1] = x1; u.u[2] = y0; u.u[3] = y1;
-          pa[kb * 2 + c] = u.v;
+#pragma unroll
+          for (int c = 0; c < 2; ++c) {
+            unsigned x0 = pk[4 * c + 0], x1 = pk[4 * c + 1];
+            unsigned y0 = pk[4 * c + 2], y1 = pk[4 * c + 3];
+            {
+              auto r0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+              x0 = r0[0]; y0 = r0[1];
+              auto r1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+              x1 = r1[0]; y1 = r1[1];
+            }
+            union { unsigned u[4]; bf16x8_t v; } u;
+            u.u[0] = x0; u.u[1] = x1; u.u[2] = y0; u.u[3] = y1;
+            pa[ps][kb * 2 + c] = u.v;
+          }
         }
       }
 
@@ -328,7 +357,10 @@ __global__ __launch_bounds__(NW * 64, 512 / (NW * 64)) void paged_prefill_mfma_v
           u.h[0] = ra[c];
           u.h[1] = rb[c];
           acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              pa[c], u.v, acc_o[dt], 0, 0, 0);
+              pa[0][c], u.v, acc_o[dt], 0, 0, 0);
+          if (WS)
+            acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                pa[PASSES - 1][c], u.v, acc_o[dt], 0, 0, 0);
         }
       }
     }
@@ -341,7 +373,17 @@ __global__ __launch_bounds__(NW * 64, 512 / (NW * 64)) void paged_prefill_mfma_v
   // NOTE: every lane stores here — in the PV output the lane indexes a d
   // column and carries ALL 32 q rows for it; q-row validity is per row
   // (q_local check below), not per lane.
-  const float l_inv_own = l_state > 0.f ? 1.f / l_state : 0.f;
+  float l_fin = l_state, o_scale = 1.f;
+  if (WS && has_sink) {
+    // the sink joins the denominator; both terms relative to the larger of
+    // the running max and the sink (log2 domain)
+    const float a2 = m2_state == -FLT_MAX ? -FLT_MAX : m2_state * sc2;
+    const float s2 = sink * LOG2E;
+    const float mf = fmaxf(a2, s2);
+    o_scale = a2 == -FLT_MAX ? 0.f : exp2f(a2 - mf);
+    l_fin = l_state * o_scale + exp2f(s2 - mf);
+  }
+  const float l_inv_own = l_fin > 0.f ? o_scale / l_fin : 0.f;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int qrow = (r & 3) + 8 * (r >> 2) + 4 * half;
@@ -363,8 +405,17 @@ static void launch_prefill_v2_ct(
     __hip_bfloat16* out, const __hip_bfloat16* q, const CT* kc, const CT* vc,
     const int* bt, const int* qsl, const int* sl, float scale, int nseq,
     int nheads, int kvh, int head_dim, int block_size, int max_blocks,
-    int max_query_len, hipStream_t stream) {
+    int max_query_len, hipStream_t stream, int window = 0, int has_sink = 0,
+    float sink = 0.f, bool ws = false) {
   if (head_dim != 128) abort();
+  if (ws) {
+    const int qtiles = (max_query_len + 255) / 256;
+    hipLaunchKernelGGL((paged_prefill_mfma_v2_kernel<128, CT, 8, true>),
+                       dim3(nseq, nheads, qtiles), dim3(512), 0, stream, out,
+                       q, kc, vc, bt, qsl, sl, scale, nheads, kvh, block_size,
+                       max_blocks, window, has_sink, sink);
+    return;
+  }
   static const int nw = [] {
     const char* e = getenv("VTA_PREFILL_WAVES");
     // measured: 8-wave/256-row wins (317/560 TF vs 302/498 for 4-wave —
@@ -373,16 +424,16 @@ static void launch_prefill_v2_ct(
   }();
   if (nw == 8) {
     const int qtiles = (max_query_len + 255) / 256;
-    hipLaunchKernelGGL((paged_prefill_mfma_v2_kernel<128, CT, 8>),
+    hipLaunchKernelGGL((paged_prefill_mfma_v2_kernel<128, CT, 8, false>),
                        dim3(nseq, nheads, qtiles), dim3(512), 0, stream, out,
                        q, kc, vc, bt, qsl, sl, scale, nheads, kvh, block_size,
-                       max_blocks);
+                       max_blocks, 0, 0, 0.f);
   } else {
     const int qtiles = (max_query_len + 127) / 128;
-    hipLaunchKernelGGL((paged_prefill_mfma_v2_kernel<128, CT, 4>),
+    hipLaunchKernelGGL((paged_prefill_mfma_v2_kernel<128, CT, 4, false>),
                        dim3(nseq, nheads, qtiles), dim3(256), 0, stream, out,
                        q, kc, vc, bt, qsl, sl, scale, nheads, kvh, block_size,
-                       max_blocks);
+                       max_blocks, 0, 0, 0.f);
   }
 }
 
@@ -405,4 +456,17 @@ void launch_paged_prefill_mfma_v2_fp8(
   launch_prefill_v2_ct<unsigned char>(out, q, kc, vc, bt, qsl, sl, scale,
                                       nseq, nheads, kvh, head_dim, block_size,
                                       max_blocks, max_query_len, stream);
+}
+
+// window + sink variant (bf16 cache, HD = 128)
+void launch_paged_prefill_mfma_v2_ws(
+    __hip_bfloat16* out, const __hip_bfloat16* q, const __hip_bfloat16* kc,
+    const __hip_bfloat16* vc, const int* bt, const int* qsl, const int* sl,
+    float scale, int nseq, int nheads, int kvh, int head_dim, int block_size,
+    int max_blocks, int max_query_len, int window, int has_sink, float sink,
+    hipStream_t stream) {
+  launch_prefill_v2_ct<__hip_bfloat16>(out, q, kc, vc, bt, qsl, sl, scale,
+                                       nseq, nheads, kvh, head_dim,
+                                       block_size, max_blocks, max_query_len,
+                                       stream, window, has_sink, sink, true);
 }

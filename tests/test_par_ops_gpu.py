@@ -218,3 +218,38 @@ def test_grouped_expert_product():
         want = ref.moe_gemm(x, w, seg, False, act)
         got = ops.moe_gemm(x.to(DEV), w.to(DEV), seg.to(DEV), gated=False, act=act)
         _close(got[:280], want[:280], torch.bfloat16, f"act {act}")
+
+
+@pytest.mark.parametrize("dim", [64, 128])
+@pytest.mark.parametrize("window,sink", [(0, 0.0), (1, 0.0), (33, None), (64, 0.0), (100, 1.0),
+                                         (257, 0.0), (5000, -1.0)])
+def test_windowed_attention_on_matrix_cores(dim, window, sink):
+    """bf16 shapes that run the MFMA kernels: windows that end inside, at the
+    edge of and beyond a key tile, portions that start mid-tile, a two-token
+    portion, single queries with a padding row."""
+    g = torch.Generator().manual_seed(8)
+    dtype = torch.bfloat16
+    heads, kv_heads, bs = 8, 2, 16
+    spec = [(300, 300), (70, 391), (2, 130), (1 + 256, 700), (5, 5)]
+    ctxs = [s[1] for s in spec]
+    kc, vc, bt = _paged(ctxs, bs, kv_heads, dim, dim, dtype, g)
+    news = torch.tensor([s[0] for s in spec])
+    qsl = torch.tensor([0] + news.cumsum(0).tolist(), dtype=torch.int32)
+    lens = torch.tensor(ctxs, dtype=torch.int32)
+    q = torch.randn(int(qsl[-1]), heads, dim, generator=g).to(dtype)
+    scale = dim ** -0.5
+    want = ref.paged_attention(q, kc, vc, bt, qsl, lens, scale, window, sink)
+    out = torch.empty(q.shape[0], heads, dim, dtype=dtype, device=DEV)
+    ops.gqa_attention_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV), qsl.to(DEV),
+                              lens.to(DEV), scale, int(news.max()), out=out, window=window,
+                              sink=sink)
+    _close(out, want, dtype, "portions")
+    lens1 = torch.tensor(ctxs + [0], dtype=torch.int32)
+    bt1 = torch.cat([bt, torch.zeros(1, bt.shape[1], dtype=torch.int32)])
+    q1 = torch.randn(len(ctxs) + 1, heads, dim, generator=g).to(dtype)
+    qsl1 = torch.arange(len(ctxs) + 2, dtype=torch.int32)
+    want1 = ref.paged_attention(q1, kc, vc, bt1, qsl1, lens1, scale, window, sink)
+    out1 = torch.empty(q1.shape[0], heads, dim, dtype=dtype, device=DEV)
+    ops.gqa_attention_decode(q1.to(DEV), kc.to(DEV), vc.to(DEV), bt1.to(DEV), lens1.to(DEV),
+                             scale, out=out1, window=window, sink=sink)
+    _close(out1, want1, dtype, "single queries")

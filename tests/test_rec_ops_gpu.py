@@ -142,13 +142,13 @@ def test_qk_norm_and_attention(dtype, dims):
     want = ref.paged_attention(q_r[:npt], kc_r, vc_r, tables[:2], qsl, sl, 0.11)
     out = torch.empty((t, heads, vdim), dtype=dtype, device=DEV)
     ops._S.paged_attention_any(out[:npt], q_r[:npt].to(DEV), kc_g, vc_g, tables[:2].to(DEV),
-                               qsl.to(DEV), sl.to(DEV), 0.11, max(news))
+                               qsl.to(DEV), sl.to(DEV), 0.11, max(news), 0, False, 0.0)
     _close(out[:npt], want, dtype, "prefill")
     sl1 = torch.tensor([lens[2], 0], dtype=torch.int32)      # second row: padding
     q1 = torch.cat([q_r[npt:], q_r[npt:]]).to(DEV)
     out1 = torch.full((2, heads, vdim), 7.0, dtype=dtype, device=DEV)
     bt1 = torch.cat([tables[2:], tables[2:]]).to(DEV)
-    ops._S.paged_attention_any(out1, q1, kc_g, vc_g, bt1, None, sl1.to(DEV), 0.11, 1)
+    ops._S.paged_attention_any(out1, q1, kc_g, vc_g, bt1, None, sl1.to(DEV), 0.11, 1, 0, False, 0.0)
     want1 = ref.paged_attention(q_r[npt:], kc_r, vc_r, tables[2:], torch.tensor([0, 1], dtype=torch.int32),
                                 sl1[:1], 0.11)
     _close(out1[:1], want1, dtype, "decode")
@@ -173,7 +173,7 @@ def test_matrix_core_attention_dispatch(dtype):
     a = torch.empty((n, heads, dim), dtype=dtype, device=DEV)
     b = torch.empty_like(a)
     ops.gqa_attention_prefill(q, kc, vc, tables, qsl, sl, 0.1, n, out=a)
-    ops._S.paged_attention_any(b, q, kc, vc, tables, qsl, sl, 0.1, n)
+    ops._S.paged_attention_any(b, q, kc, vc, tables, qsl, sl, 0.1, n, 0, False, 0.0)
     _close(a, b, dtype, "prefill dispatch")
     ops.gqa_attention_decode(q[-1:], kc, vc, tables, sl, 0.1, out=a[:1])
     _close(a[:1], b[-1:], dtype, "decode dispatch")

@@ -123,18 +123,31 @@ def model_config_from_json(model: str, hf: dict) -> ModelConfig:
         max_model_len=int(hf.get("max_len", _DEFAULT_MAX_LEN)),
         tie_word_embeddings=False,
         dtype=torch.bfloat16,
-        num_experts=max((int(m["router"]["experts"]) for m in moe), default=0),
-        num_experts_per_tok=max((int(m["router"]["top"]) for m in moe), default=0),
+        # num_experts stays 0: that field describes the mixtral expert layout
+        # (and gates its capture rules); the routed layers here are shape-static
         hf_config=hf,
     )
 
 
 def native_extensions(cfg: ModelConfig) -> list[str]:
-    """Stream ops, rotation + cache write, attention, gates and router live in
-    the sequence extension; latent attention has its own."""
+    """Stream ops, rotation + cache write, any-shape attention, gates and
+    router live in the sequence extension; latent attention has its own; the
+    MFMA attention kernels (alone, without the rest of their extension) are
+    needed when an attention mixer has a shape they take."""
     need = ["_C_seq"]
-    if any(e.get("type") == "latent_attention" for e in cfg.hf_config["layers"]):
+    layers = cfg.hf_config["layers"]
+    if any(e.get("type") == "latent_attention" for e in layers):
         need.append("_C_lat")
+    for e in layers:
+        if e.get("type") != "attention":
+            continue
+        a = e["mixer"]
+        dim = int(a["dim"])
+        if ops.windowed_attention_uses_matrix_cores(
+                cfg.dtype, int(a["heads"]), int(a.get("kv_heads", a["heads"])), dim,
+                int(a.get("vdim", dim))):
+            need.append("_C_attn")
+            break
     return need
 
 

@@ -752,9 +752,24 @@ def _matrix_core_attention_fits(q: torch.Tensor, k_cache: torch.Tensor,
 
 
 def _windowed_matrix_core_fits(q: torch.Tensor, k_cache: torch.Tensor,
-                               v_cache: torch.Tensor) -> bool:
-    """No matrix-core kernel takes a window or a sink yet."""
-    return False
+                               v_cache: torch.Tensor, single: bool) -> bool:
+    """The window + sink variants of the MFMA kernels take bf16, equal key and
+    value size of 128 (single queries: also 64), up to 8 query heads per key
+    head."""
+    if _attn_ext() is None or _FORCE_REFERENCE or q.dtype != torch.bfloat16:
+        return False
+    d = q.shape[-1]
+    group = q.shape[1] // k_cache.shape[2]
+    return (d in ((64, 128) if single else (128,)) and v_cache.shape[-1] == d
+            and 1 <= group <= 8 and q.shape[1] == group * k_cache.shape[2]
+            and q.is_contiguous())
+
+
+def windowed_attention_uses_matrix_cores(dtype: torch.dtype, heads: int, kv_heads: int,
+                                         dim: int, vdim: int) -> bool:
+    """Shape test of the above without tensors (which extensions a model needs)."""
+    return (dtype == torch.bfloat16 and dim == vdim and dim in (64, 128)
+            and heads % kv_heads == 0 and 1 <= heads // kv_heads <= 8)
 
 
 def attention_uses_matrix_cores(dtype: torch.dtype, heads: int, kv_heads: int,
@@ -775,11 +790,14 @@ def gqa_attention_prefill(q, k_cache, v_cache, block_tables, query_start_loc,
     sizes, value size unlike the key size) on the any-shape kernel."""
     if q.numel() and _native_seq(q):
         if window > 0 or sink is not None:
-            if _windowed_matrix_core_fits(q, k_cache, v_cache):
-                _S.windowed_attention_mfma(out, q, k_cache, v_cache, block_tables,
-                                           query_start_loc, seq_lens, float(scale),
-                                           int(max_query_len), int(window),
-                                           sink is not None, float(sink or 0.0))
+            if _windowed_matrix_core_fits(q, k_cache, v_cache, single=False):
+                dst = out if out.is_contiguous() else torch.empty_like(q)
+                _attn_ext().windowed_attention_prefill(
+                    dst, q, k_cache, v_cache, block_tables, query_start_loc, seq_lens,
+                    float(scale), int(max_query_len), int(window), sink is not None,
+                    float(sink or 0.0))
+                if dst is not out:
+                    out.copy_(dst)
                 return out
             _S.paged_attention_any(out, q, k_cache, v_cache, block_tables,
                                    query_start_loc, seq_lens, float(scale),
@@ -811,11 +829,13 @@ def gqa_attention_decode(q, k_cache, v_cache, block_tables, seq_lens, scale,
     zeros)."""
     if q.numel() and _native_seq(q):
         if window > 0 or sink is not None:
-            if _windowed_matrix_core_fits(q, k_cache, v_cache):
-                _S.windowed_attention_mfma(out, q, k_cache, v_cache, block_tables,
-                                           None, seq_lens, float(scale), 1,
-                                           int(window), sink is not None,
-                                           float(sink or 0.0))
+            if _windowed_matrix_core_fits(q, k_cache, v_cache, single=True):
+                dst = out if out.is_contiguous() else torch.empty_like(q)
+                _attn_ext().windowed_attention_decode(
+                    dst, q, k_cache, v_cache, block_tables, seq_lens, float(scale),
+                    int(window), sink is not None, float(sink or 0.0))
+                if dst is not out:
+                    out.copy_(dst)
                 return out
             _S.paged_attention_any(out, q, k_cache, v_cache, block_tables, None,
                                    seq_lens, float(scale), 1, int(window),
