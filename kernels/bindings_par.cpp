@@ -28,6 +28,10 @@ void launch_moe_route(float*, float*, int*, float*, const float*, const float*,
 template <typename T>
 void launch_moe_combine(T*, const T*, const int*, const int*, const float*, int,
                         int, int, int, hipStream_t);
+int moe_sort_max_experts();
+template <typename T>
+void launch_moe_sort(T*, int*, int*, int*, const T*, long, const int*, int, int,
+                     int, int, hipStream_t);
 void launch_moe_gemm(__hip_bfloat16*, const __hip_bfloat16*,
                      const __hip_bfloat16*, const int*, int, int, int, int, int,
                      hipStream_t);
@@ -256,6 +260,29 @@ void moe_combine(torch::Tensor out, torch::Tensor ye, torch::Tensor pos,
   });
 }
 
+void moe_sort(torch::Tensor xs, torch::Tensor pos, torch::Tensor seg,
+              torch::Tensor scratch, torch::Tensor h, torch::Tensor ids,
+              int64_t num_real) {
+  check_i32(ids, "ids");
+  check_i32(pos, "pos");
+  check_i32(seg, "seg");
+  check_i32(scratch, "scratch");
+  TORCH_CHECK(h.is_cuda() && h.dim() == 2 && h.stride(1) == 1 && ids.dim() == 2 &&
+              ids.size(0) == h.size(0));
+  const int tokens = h.size(0), width = h.size(1), top = ids.size(1);
+  TORCH_CHECK(num_real >= 1 && num_real <= moe_sort_max_experts(), "number of experts");
+  TORCH_CHECK(pos.sizes() == ids.sizes() && seg.numel() == num_real + 1 &&
+              scratch.numel() == 2 * num_real);
+  TORCH_CHECK(xs.is_contiguous() && xs.dim() == 2 && xs.size(0) == (long)tokens * top &&
+              xs.size(1) == width && xs.scalar_type() == h.scalar_type());
+  if (tokens == 0) return;
+  DISPATCH_F32_BF16(h.scalar_type(), {
+    launch_moe_sort<scalar_t>(ptr<scalar_t>(xs), ptr<int>(pos), ptr<int>(seg),
+                              ptr<int>(scratch), ptr<scalar_t>(h), (long)h.stride(0),
+                              ptr<int>(ids), tokens, top, (int)num_real, width, stream());
+  });
+}
+
 // mode 0: plain, 1: silu(first half) * second half, 2: squared relu
 void moe_gemm(torch::Tensor y, torch::Tensor x, torch::Tensor w,
               torch::Tensor seg_off, int64_t mode) {
@@ -288,5 +315,6 @@ void register_par_ops(pybind11::module& m) {
   m.def("relu2", &relu2);
   m.def("moe_route", &moe_route);
   m.def("moe_combine", &moe_combine);
+  m.def("moe_sort", &moe_sort);
   m.def("moe_gemm", &moe_gemm);
 }

@@ -12,6 +12,8 @@
 //   moe_route                 softmax over experts, corrected top-k choice,
 //                             normalised weights, identity experts summed
 //   moe_combine               weighted gather-sum of expert outputs per token
+//   moe_sort                  token-expert pairs grouped by expert: segment
+//                             offsets, each pair's row, the gathered input rows
 //
 // All memory-bound; norm statistics, angles, sigmoids, router arithmetic and
 // the stream are f32 whatever the storage type.
@@ -193,6 +195,78 @@ __global__ __launch_bounds__(256) void rope_kv_cache_write_kernel(
     const float other = ScalarOps<T>::to_f32(src[partner]);
     dst[c] = ScalarOps<T>::from_f32(first ? self * cs - other * sn : self * cs + other * sn);
   }
+}
+
+// Vector variant: `lph` lanes per head, each owning 16 bytes (V elements) of
+// it; sizes and strides are multiples of V, for half-split pairs the half is a
+// multiple of V too (the lane of the first half also loads, rotates and stores
+// the partner chunk).  grid (tokens, ceil(units / units_per_block)).
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kv_cache_write_vec_kernel(
+    T* __restrict__ q_out, const T* __restrict__ q, long q_st,
+    const T* __restrict__ k, long k_st, const T* __restrict__ v, long v_st,
+    const long* __restrict__ positions, const float* __restrict__ inv_freq,
+    int half, int interleaved, float mag, T* __restrict__ k_cache,
+    T* __restrict__ v_cache, const long* __restrict__ slot_mapping, int heads,
+    int kv_heads, int dim, int vdim, int lph, int upb) {
+  constexpr int V = Vec16<T>::kElems;
+  const long t = blockIdx.x;
+  const int u_in = threadIdx.x / lph;
+  const int l = threadIdx.x - u_in * lph;
+  const int unit = blockIdx.y * upb + u_in;
+  if (u_in >= upb || unit >= heads + 2 * kv_heads) return;
+  const long slot = slot_mapping[t];
+  const int c0 = l * V;
+  if (unit >= heads + kv_heads) {
+    if (slot < 0 || c0 >= vdim) return;
+    const int g = unit - heads - kv_heads;
+    store16(v_cache + (slot * kv_heads + g) * vdim + c0,
+            load16(v + t * v_st + (long)g * vdim + c0));
+    return;
+  }
+  if (c0 >= dim) return;
+  const bool is_q = unit < heads;
+  const int hh = is_q ? unit : unit - heads;
+  if (!is_q && slot < 0) return;
+  const T* src = is_q ? q + t * q_st + (long)hh * dim : k + t * k_st + (long)hh * dim;
+  T* dst = is_q ? q_out + (t * heads + hh) * dim : k_cache + (slot * kv_heads + hh) * dim;
+  const int rot = 2 * half;
+  Vec16<T> a = load16(src + c0);
+  if (c0 >= rot) {
+    store16(dst + c0, a);
+    return;
+  }
+  const float pos = (float)positions[t];
+  if (interleaved) {
+#pragma unroll
+    for (int i = 0; i < V / 2; ++i) {
+      float sn, cs;
+      sincosf(pos * inv_freq[c0 / 2 + i], &sn, &cs);
+      sn *= mag;
+      cs *= mag;
+      const float x0 = ScalarOps<T>::to_f32(a.data[2 * i]);
+      const float x1 = ScalarOps<T>::to_f32(a.data[2 * i + 1]);
+      a.data[2 * i] = ScalarOps<T>::from_f32(x0 * cs - x1 * sn);
+      a.data[2 * i + 1] = ScalarOps<T>::from_f32(x1 * cs + x0 * sn);
+    }
+    store16(dst + c0, a);
+    return;
+  }
+  if (c0 >= half) return;   // written by the lane that owns the first half
+  Vec16<T> b = load16(src + c0 + half);
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    float sn, cs;
+    sincosf(pos * inv_freq[c0 + i], &sn, &cs);
+    sn *= mag;
+    cs *= mag;
+    const float x0 = ScalarOps<T>::to_f32(a.data[i]);
+    const float x1 = ScalarOps<T>::to_f32(b.data[i]);
+    a.data[i] = ScalarOps<T>::from_f32(x0 * cs - x1 * sn);
+    b.data[i] = ScalarOps<T>::from_f32(x1 * cs + x0 * sn);
+  }
+  store16(dst + c0, a);
+  store16(dst + c0 + half, b);
 }
 
 // out[t, h*D + d] = o[t, h, d] * sigmoid(gate); n counts groups of S elements.
@@ -382,11 +456,116 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(
   }
 }
 
+// Grouping token-expert pairs by expert without a sort: count the pairs of
+// each real expert, turn the counts into segment offsets, hand every pair the
+// next free row of its expert's segment, copy the token's input row there.
+// Which row of its segment a pair gets depends on the order the atomics land
+// in; the grouped product computes every row on its own, so the values do not.
+constexpr int MS_MAX = 512;   // real experts
+
+__global__ __launch_bounds__(256) void moe_count_kernel(
+    int* __restrict__ counts, const int* __restrict__ ids, int npairs, int num_real) {
+  __shared__ int hist[MS_MAX];
+  for (int e = threadIdx.x; e < num_real; e += blockDim.x) hist[e] = 0;
+  __syncthreads();
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < npairs;
+       i += gridDim.x * blockDim.x) {
+    const int e = ids[i];
+    if (e < num_real) atomicAdd(&hist[e], 1);
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < num_real; e += blockDim.x)
+    if (hist[e]) atomicAdd(&counts[e], hist[e]);
+}
+
+__global__ __launch_bounds__(256) void moe_place_kernel(
+    int* __restrict__ pos, int* __restrict__ seg, int* __restrict__ cursor,
+    const int* __restrict__ counts, const int* __restrict__ ids, int npairs,
+    int num_real) {
+  __shared__ int seg_s[MS_MAX + 1];
+  __shared__ int hist[MS_MAX];   // this round's pairs of the workgroup per expert
+  __shared__ int base[MS_MAX];   // where the workgroup's run starts in the segment
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int e = 0; e < num_real; ++e) {
+      seg_s[e] = run;
+      run += counts[e];
+    }
+    seg_s[num_real] = run;
+  }
+  __syncthreads();
+  if (blockIdx.x == 0)
+    for (int e = threadIdx.x; e <= num_real; e += blockDim.x) seg[e] = seg_s[e];
+  // rounds of one pair per thread: rank the pairs inside the workgroup through
+  // LDS, reserve one run per (workgroup, expert) with a single global atomic
+  const int stride = gridDim.x * blockDim.x;
+  const int rounds = (npairs + stride - 1) / stride;
+  for (int r = 0; r < rounds; ++r) {
+    const int i = r * stride + blockIdx.x * blockDim.x + threadIdx.x;
+    for (int e = threadIdx.x; e < num_real; e += blockDim.x) hist[e] = 0;
+    __syncthreads();
+    int e = num_real, local = 0;
+    if (i < npairs) {
+      e = ids[i];
+      if (e < num_real) local = atomicAdd(&hist[e], 1);
+    }
+    __syncthreads();
+    for (int x = threadIdx.x; x < num_real; x += blockDim.x)
+      if (hist[x]) base[x] = atomicAdd(&cursor[x], hist[x]);
+    __syncthreads();
+    if (i < npairs) pos[i] = (e < num_real) ? seg_s[e] + base[e] + local : 0;
+    __syncthreads();   // hist and base are reused by the next round
+  }
+}
+
+// one workgroup per token: its row goes to the rows of its real experts
+template <typename T>
+__global__ __launch_bounds__(256) void moe_gather_kernel(
+    T* __restrict__ xs, const T* __restrict__ h, long h_st,
+    const int* __restrict__ pos, const int* __restrict__ ids, int top,
+    int num_real, int width, int vec) {
+  const long t = blockIdx.x;
+  const T* src = h + t * h_st;
+  if (vec) {
+    constexpr int V = Vec16<T>::kElems;
+    for (int c = threadIdx.x * V; c < width; c += blockDim.x * V) {
+      const Vec16<T> v = load16(src + c);
+      for (int k = 0; k < top; ++k)
+        if (ids[t * top + k] < num_real)
+          store16(xs + (long)pos[t * top + k] * width + c, v);
+    }
+  } else {
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+      const T v = src[c];
+      for (int k = 0; k < top; ++k)
+        if (ids[t * top + k] < num_real) xs[(long)pos[t * top + k] * width + c] = v;
+    }
+  }
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------
 // launchers
 // ---------------------------------------------------------------------------
+
+int moe_sort_max_experts() { return MS_MAX; }
+
+// counts_cursor: 2 * num_real zeros (counts, then the per-expert cursors)
+template <typename T>
+void launch_moe_sort(T* xs, int* pos, int* seg, int* counts_cursor, const T* h,
+                     long h_st, const int* ids, int tokens, int top, int num_real,
+                     int width, hipStream_t s) {
+  const int npairs = tokens * top;
+  const int blocks = grid_for(npairs, 256) > 1024 ? 1024 : grid_for(npairs, 256);
+  moe_count_kernel<<<blocks, 256, 0, s>>>(counts_cursor, ids, npairs, num_real);
+  moe_place_kernel<<<blocks, 256, 0, s>>>(pos, seg, counts_cursor + num_real,
+                                           counts_cursor, ids, npairs, num_real);
+  constexpr int V = Vec16<T>::kElems;
+  const int vec = width % V == 0 && h_st % V == 0 && al(xs, 16) && al(h, 16);
+  moe_gather_kernel<T><<<tokens, 256, 0, s>>>(xs, h, h_st, pos, ids, top, num_real,
+                                             width, vec);
+}
 
 template <typename T>
 void launch_stream_add_rms_norm_pair(float* x, const T* a, const T* b,
@@ -413,6 +592,22 @@ void launch_rope_kv_cache_write(T* q_out, const T* q, long q_st, const T* k,
                                 int heads, int kv_heads, int dim, int vdim,
                                 hipStream_t s) {
   const int units = heads + 2 * kv_heads;
+  constexpr int V = Vec16<T>::kElems;
+  const int rot = 2 * half;
+  const int big = dim > vdim ? dim : vdim;
+  const bool vec = dim % V == 0 && vdim % V == 0 && big / V <= 256 && q_st % V == 0 &&
+                   k_st % V == 0 && v_st % V == 0 && rot % V == 0 &&
+                   (interleaved || half % V == 0) && al(q_out, 16) && al(q, 16) &&
+                   al(k, 16) && al(v, 16) && al(k_cache, 16) && al(v_cache, 16);
+  if (vec) {
+    const int lph = big / V;
+    const int upb = 256 / lph;
+    dim3 vgrid(tokens, (units + upb - 1) / upb);
+    rope_kv_cache_write_vec_kernel<T><<<vgrid, 256, 0, s>>>(
+        q_out, q, q_st, k, k_st, v, v_st, positions, inv_freq, half, interleaved,
+        mag, k_cache, v_cache, slot_mapping, heads, kv_heads, dim, vdim, lph, upb);
+    return;
+  }
   dim3 grid(tokens, (units + 3) / 4);
   rope_kv_cache_write_kernel<T><<<grid, 256, 0, s>>>(
       q_out, q, q_st, k, k_st, v, v_st, positions, inv_freq, half, interleaved,
@@ -476,6 +671,8 @@ void launch_moe_combine(T* out, const T* ye, const int* pos, const int* ids,
 }
 
 #define INSTANTIATE(T)                                                           \
+  template void launch_moe_sort<T>(T*, int*, int*, int*, const T*, long,         \
+                                   const int*, int, int, int, int, hipStream_t); \
   template void launch_stream_add_rms_norm_pair<T>(                              \
       float*, const T*, const T*, const float*, const T*, const float*,          \
       const float*, float, int, int, T*, T*, hipStream_t);                       \

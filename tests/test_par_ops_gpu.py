@@ -253,3 +253,28 @@ def test_windowed_attention_on_matrix_cores(dim, window, sink):
     ops.gqa_attention_decode(q1.to(DEV), kc.to(DEV), vc.to(DEV), bt1.to(DEV), lens1.to(DEV),
                              scale, out=out1, window=window, sink=sink)
     _close(out1, want1, dtype, "single queries")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("t,top,real,extra,width", [(37, 3, 5, 2, 64), (300, 4, 16, 4, 40),
+                                                    (1, 2, 2, 0, 7), (64, 1, 1, 3, 128)])
+def test_pairs_grouped_by_expert(dtype, t, top, real, extra, width):
+    g = torch.Generator().manual_seed(9)
+    # distinct experts per token, as a router gives them
+    ids = torch.stack([torch.randperm(real + extra, generator=g)[:top] for _ in range(t)]).to(torch.int32)
+    h = torch.randn(t, width + 8, generator=g).to(dtype)[:, 8:]      # a column slice
+    xs, pos, seg = ops.moe_sort(ids.to(DEV), real, h.to(DEV)[:, :] if width % 8 else h.to(DEV))
+    _, _, seg_r = ref.moe_sort(ids, real, h)
+    assert torch.equal(seg.cpu(), seg_r)
+    xs, pos, seg = xs.cpu(), pos.cpu().long(), seg.cpu().tolist()
+    taken = set()
+    for i in range(t):
+        for k in range(top):
+            e = int(ids[i, k])
+            if e >= real:
+                continue
+            p = int(pos[i, k])
+            assert seg[e] <= p < seg[e + 1] and p not in taken     # its own row of its segment
+            taken.add(p)
+            assert torch.equal(xs[p], h[i])
+    assert len(taken) == seg[-1]

@@ -164,9 +164,12 @@ class LatentAttention(nn.Module):
         self.q_proj = ColumnParallelLinear(width, heads * (dim + rot_dim), dtype=dtype)
         self.o_proj = RowParallelLinear(heads * vdim, width, dtype=dtype)
         if kv_owner:
-            # replicated on every rank: the latent is shared by all heads
+            # replicated on every rank: the latent is shared by all heads.  With a
+            # head gate this rank's gate rows follow the down-projection's, so
+            # that one product yields both
             self.dkv_weight = nn.Parameter(
-                torch.empty(rank + rot_dim, width, dtype=dtype).normal_(0.0, 0.02),
+                torch.empty(rank + rot_dim + (self.heads if head_gate else 0), width,
+                            dtype=dtype).normal_(0.0, 0.02),
                 requires_grad=False)
             self.dkv_norm = _f32_param(rank, fill=1.0)
         # [H, dim, rank] and [H, rank, vdim] for the batched fold / unfold
@@ -182,10 +185,11 @@ class LatentAttention(nn.Module):
         self.register_buffer(
             "inv_freq", torch.tensor(freqs, dtype=torch.float64).to(torch.float32),
             persistent=False)
-        # this rank's heads' rows of the gate projection
+        self.head_gate = head_gate
+        # a layer without a down-projection of its own keeps its gate rows apart
         self.gate_weight = (
             nn.Parameter(torch.empty(self.heads, width, dtype=dtype).normal_(0.0, 0.02),
-                         requires_grad=False) if head_gate else None)
+                         requires_grad=False) if head_gate and not kv_owner else None)
 
     # -- weights -----------------------------------------------------------
     def load(self, q, dkv, dkv_norm, uk, uv, sink, o, gate=None) -> None:
@@ -195,7 +199,10 @@ class LatentAttention(nn.Module):
         if self.gate_weight is not None:
             self.gate_weight.data.copy_(gate[r * h:(r + 1) * h].to(self.dtype))
         if self.kv_owner:
-            self.dkv_weight.data.copy_(dkv.to(self.dtype))
+            n = self.rank + self.rot_dim
+            self.dkv_weight.data[:n].copy_(dkv.to(self.dtype))
+            if self.head_gate:
+                self.dkv_weight.data[n:].copy_(gate[r * h:(r + 1) * h].to(self.dtype))
             self.dkv_norm.data.copy_(dkv_norm.float())
         uk = uk.view(-1, self.dim, self.rank)[r * h:(r + 1) * h]
         uv = uv.view(-1, self.vdim, self.rank)[r * h:(r + 1) * h]
@@ -212,8 +219,11 @@ class LatentAttention(nn.Module):
         q = self.q_proj(h).view(t, nh, d + r)
         ops.rope_partial(q, positions, self.inv_freq, d, self.rot_dims,
                          self.rot_interleaved, self.rot_mag)
+        g = None
         if self.kv_owner:
             dkv = ops.linear(h, self.dkv_weight)
+            if self.head_gate:
+                dkv, g = dkv[:, :rank + r], dkv[:, rank + r:]
             ops.latent_kv_write(dkv, self.dkv_norm, self.eps, positions,
                                 self.inv_freq, self.rot_dims, cache,
                                 meta.slot_mapping, self.rot_interleaved, self.rot_mag)
@@ -235,9 +245,10 @@ class LatentAttention(nn.Module):
                 meta.decode_seq_lens, self.scale, self.window, self.sink,
                 out=o_view[npt:])
         o = torch.bmm(o_lat, self.uv_t)                    # [H, T, vdim]
-        if self.gate_weight is not None:
+        if self.head_gate:
             # gate and the [H, T] -> [T, H] regrouping in one pass
-            g = ops.linear(h, self.gate_weight)            # [T, H]
+            if g is None:
+                g = ops.linear(h, self.gate_weight)        # [T, H]
             return self.o_proj(ops.sigmoid_gate_mul(o.transpose(0, 1), g))
         return self.o_proj(o.transpose(0, 1).reshape(t, nh * self.vdim))
 
@@ -821,17 +832,9 @@ class RoutedExperts(nn.Module):
         if not self.grouped:
             u = ops.linear(h, self.up.view(self.experts * self.ff, self.width))
             return ops.linear(ops.relu2(u, None, dense), self.down), ident
-        t, top, ne = h.shape[0], self.top, self.experts
-        # pairs sorted by expert (identity experts sort last and are skipped)
-        flat = ids.reshape(-1).long()
-        order = torch.argsort(flat, stable=True)
-        pos = torch.empty_like(order)
-        pos[order] = torch.arange(t * top, device=h.device)
-        counts = torch.zeros(ne + self.identity, dtype=torch.int32, device=h.device)
-        counts.scatter_add_(0, flat, torch.ones_like(flat, dtype=torch.int32))
-        seg = torch.zeros(ne + 1, dtype=torch.int32, device=h.device)
-        seg[1:] = counts[:ne].cumsum(0).to(torch.int32)
-        xs = h[torch.div(order, top, rounding_mode="floor")]
+        ne = self.experts
+        # pairs grouped by expert (identity experts get no row)
+        xs, pos, seg = ops.moe_sort(ids, ne, h)
         a = ops.moe_gemm(xs, self.up, seg, gated=False, act="relu2")
         ye = ops.moe_gemm(a, self.down, seg, gated=False)
-        return ops.moe_combine(ye, pos.view(t, top).to(torch.int32), ids, w, ne), ident
+        return ops.moe_combine(ye, pos, ids, w, ne), ident

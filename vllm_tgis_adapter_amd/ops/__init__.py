@@ -1011,3 +1011,22 @@ def moe_combine(ye: torch.Tensor, pos: torch.Tensor, ids: torch.Tensor,
         _S.moe_combine(out, ye, pos, ids, weights, int(num_real))
         return out
     return reference.moe_combine(ye, pos, ids, weights, num_real)
+
+
+def moe_sort(ids: torch.Tensor, num_real: int, h: torch.Tensor):
+    """Group the token-expert pairs ids [T, top] by expert.  Returns (xs
+    [T * top, W]: h's rows gathered so that expert e's pairs fill rows seg[e] ..
+    seg[e+1], pos [T, top] int32: the row of each pair (0 for identity experts,
+    ids >= num_real, which get no row), seg [num_real + 1] int32).  Rows past
+    seg[-1] are left unwritten.  The order of the pairs inside a segment is
+    not specified."""
+    if h.numel() and _native_seq(h):
+        t, top = ids.shape
+        dev = h.device
+        xs = torch.empty((t * top, h.shape[1]), dtype=h.dtype, device=dev)
+        pos = torch.empty((t, top), dtype=torch.int32, device=dev)
+        seg = torch.empty((num_real + 1,), dtype=torch.int32, device=dev)
+        scratch = torch.zeros((2 * num_real,), dtype=torch.int32, device=dev)
+        _S.moe_sort(xs, pos, seg, scratch, h, ids, int(num_real))
+        return xs, pos, seg
+    return reference.moe_sort(ids, num_real, h)

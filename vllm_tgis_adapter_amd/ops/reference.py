@@ -715,3 +715,19 @@ def moe_gemm(x: torch.Tensor, w: torch.Tensor, seg_off: torch.Tensor, gated: boo
             y = torch.clamp(y, min=0.0) ** 2
         out[a:b] = y.to(x.dtype)
     return out
+
+
+def moe_sort(ids: torch.Tensor, num_real: int, h: torch.Tensor):
+    """Token-expert pairs grouped by expert (stable): gathered rows, each
+    pair's row, segment offsets of the real experts."""
+    t, top = ids.shape
+    flat = ids.reshape(-1).long()
+    order = torch.argsort(flat, stable=True)
+    pos = torch.empty_like(order)
+    pos[order] = torch.arange(t * top, device=ids.device)
+    counts = torch.bincount(flat, minlength=num_real)[:num_real]
+    seg = torch.zeros(num_real + 1, dtype=torch.int32, device=ids.device)
+    seg[1:] = counts.cumsum(0).to(torch.int32)
+    xs = h[torch.div(order, top, rounding_mode="floor")]
+    pos = torch.where(flat < num_real, pos, torch.zeros_like(pos))
+    return xs, pos.view(t, top).to(torch.int32), seg
