@@ -483,7 +483,7 @@ __global__ __launch_bounds__(256) void moe_place_kernel(
     const int* __restrict__ counts, const int* __restrict__ ids, int npairs,
     int num_real) {
   __shared__ int seg_s[MS_MAX + 1];
-  __shared__ int hist[MS_MAX];   // this round's pairs of the workgroup per expert
+  __shared__ int hist[MS_MAX];   // the workgroup's pairs of this pass, per expert
   __shared__ int base[MS_MAX];   // where the workgroup's run starts in the segment
   if (threadIdx.x == 0) {
     int run = 0;
@@ -496,11 +496,11 @@ __global__ __launch_bounds__(256) void moe_place_kernel(
   __syncthreads();
   if (blockIdx.x == 0)
     for (int e = threadIdx.x; e <= num_real; e += blockDim.x) seg[e] = seg_s[e];
-  // rounds of one pair per thread: rank the pairs inside the workgroup through
+  // passes of one pair per thread: rank the pairs inside the workgroup through
   // LDS, reserve one run per (workgroup, expert) with a single global atomic
   const int stride = gridDim.x * blockDim.x;
-  const int rounds = (npairs + stride - 1) / stride;
-  for (int r = 0; r < rounds; ++r) {
+  const int passes = (npairs + stride - 1) / stride;
+  for (int r = 0; r < passes; ++r) {
     const int i = r * stride + blockIdx.x * blockDim.x + threadIdx.x;
     for (int e = threadIdx.x; e < num_real; e += blockDim.x) hist[e] = 0;
     __syncthreads();
@@ -514,7 +514,7 @@ __global__ __launch_bounds__(256) void moe_place_kernel(
       if (hist[x]) base[x] = atomicAdd(&cursor[x], hist[x]);
     __syncthreads();
     if (i < npairs) pos[i] = (e < num_real) ? seg_s[e] + base[e] + local : 0;
-    __syncthreads();   // hist and base are reused by the next round
+    __syncthreads();   // hist and base are reused by the next pass
   }
 }
 

@@ -6,20 +6,23 @@ parallel blocks with two norms,
 both RMS norms (plain weight) of the same x, so they share one statistic.  The
 mixer of a layer is one of
 
-  attention         grouped-query softmax attention with rotary positions on the
-                    first rot.dims dims of each head (interleaved pairs, YaRN
-                    frequency scaling), whose values are the keys as projected
-                    (before rotation); a sliding window; a softmax denominator
-                    with one extra 1 (a sink of score 0 that has no value); the
-                    concatenated heads times sigmoid(W_g h) before W_o
+  attention         grouped-query softmax attention; rot.dims leading dims of
+                    every head are rotated (neighbouring dims form a pair,
+                    frequencies stretched the YaRN way); there is no value
+                    projection, the unrotated key projections serve as values;
+                    keys further back than mask.size - 1 positions are masked;
+                    the softmax denominator is 1 + sum(exp(s)), i.e. a sink
+                    with logit 0 and no value; W_o reads the heads multiplied
+                    elementwise by sigmoid(W_g h)
   latent_attention  causal attention over one cached latent row per token
                     (RMS-normed latent + one rotated key part shared by all
                     heads), ordinary softmax, head h's output times
                     sigmoid(W_g h)_h
 
 and the feed-forward is dense (squared relu, biases), a mixture of small
-squared-relu experts plus identity experts behind a softmax router with a
-choice correction, or absent.  The head is the final RMS norm and a linear map.
+squared-relu experts plus identity experts (output = input) behind a softmax
+router (top-k picked on score + correction, weighted by the renormalised plain
+scores), or absent.  The head is the final RMS norm and a linear map.
 
 Sizes and constants all come from config.json:
 
