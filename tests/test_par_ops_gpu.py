@@ -278,3 +278,52 @@ def test_pairs_grouped_by_expert(dtype, t, top, real, extra, width):
             taken.add(p)
             assert torch.equal(xs[p], h[i])
     assert len(taken) == seg[-1]
+
+
+@pytest.mark.parametrize("dim", [64, 128])
+@pytest.mark.parametrize("n_new", [1, 2, 70])
+@pytest.mark.parametrize("window", [33, 64, 100, 257, 0])
+def test_window_edge_on_matrix_cores(dim, n_new, window):
+    """bf16 MFMA kernels: one key that the last query points at, with a value of
+    100, placed just inside and just outside the window, at the sequence's
+    start and at tile borders; everything else is small noise."""
+    import math
+
+    ctx, bs, dtype = 300, 16, torch.bfloat16
+    nb = (ctx + bs - 1) // bs
+    table = list(range(nb - 1, -1, -1))
+    places = {0, ctx - 1, 63, 64, 255, 256}
+    if window:
+        places |= {ctx - window, ctx - window - 1, ctx - window + 1}
+    for at in sorted(places):
+        g = torch.Generator().manual_seed(at)
+        k = torch.randn(ctx, 1, dim, generator=g) * 0.02
+        v = torch.randn(ctx, 1, dim, generator=g) * 0.02
+        q = torch.randn(n_new, 2, dim, generator=g) * 0.02
+        direction = torch.ones(dim) / math.sqrt(dim)
+        k[at, 0] = 8.0 * direction
+        v[at, 0] = 100.0
+        q[-1, :] = 8.0 * direction
+        k, v, q = k.to(dtype), v.to(dtype), q.to(dtype)
+        kc = torch.zeros(nb, bs, 1, dim, dtype=dtype)
+        vc = torch.zeros(nb, bs, 1, dim, dtype=dtype)
+        for p in range(ctx):
+            kc[table[p // bs], p % bs] = k[p]
+            vc[table[p // bs], p % bs] = v[p]
+        i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+        out = torch.empty(n_new, 2, dim, dtype=dtype, device=DEV)
+        if n_new > 1:
+            ops.gqa_attention_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), i32([table]),
+                                      i32([0, n_new]), i32([ctx]), 1.0, n_new, out=out,
+                                      window=window, sink=0.0)
+        else:
+            ops.gqa_attention_decode(q.to(DEV), kc.to(DEV), vc.to(DEV), i32([table]),
+                                     i32([ctx]), 1.0, out=out, window=window, sink=0.0)
+        lo = max(0, ctx - window) if window else 0
+        s = k[lo:ctx, 0].double() @ q[-1, 0].double()
+        e = torch.exp(s)
+        want = (e / (1.0 + e.sum())) @ v[lo:ctx, 0].double()
+        seen = at >= lo
+        assert (float(want.abs().max()) > 50.0) == seen
+        got = out[-1, 0].double().cpu()
+        assert float((got - want).abs().max()) < 0.6, f"spike at {at}: {got[:3]} vs {want[:3]}"
