@@ -646,7 +646,12 @@ def _arch_measure(mc, args, device: str, batch: int, prompt_len: int, steps: int
             engine.abort_request(rid)
         while engine.has_unfinished():
             engine.step()
+    # the engine holds reference cycles (graphs, caches): collect them now, or
+    # the next model's decode steps share the process with its leftovers
     del engine
+    import gc
+
+    gc.collect()
     if device == "cuda":
         torch.cuda.empty_cache()
     return res

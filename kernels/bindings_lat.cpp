@@ -17,7 +17,7 @@ void launch_latent_attn_mfma(__hip_bfloat16*, long, long,
                              const __hip_bfloat16*, long, long,
                              const __hip_bfloat16*, const int*, int, const int*,
                              const int*, int, const float*, float, int, int,
-                             int, int, int, int, int, float*, float*,
+                             int, int, int, int, int, int, float*, float*,
                              hipStream_t);
 int latent_decode_num_splits(int nseq, int heads, int max_keys);
 
@@ -65,7 +65,7 @@ void latent_attention_common(torch::Tensor& out, torch::Tensor& q_lat,
                              torch::Tensor& seq_lens, double scale,
                              int64_t window,
                              c10::optional<torch::Tensor>& sinks,
-                             int max_q, bool allow_mfma) {
+                             int max_q, bool allow_mfma, bool two_term) {
   TORCH_CHECK(q_lat.is_cuda() && q_lat.dim() == 3 && q_rot.dim() == 3 &&
               out.dim() == 3);
   TORCH_CHECK(q_lat.stride(2) == 1 && q_rot.stride(2) == 1 && out.stride(2) == 1);
@@ -120,7 +120,7 @@ void latent_attention_common(torch::Tensor& out, torch::Tensor& q_lat,
         q_rot.stride(1), ptr<bf>(cache), ptr<int>(block_tables),
         (int)block_tables.stride(0), qsl, ptr<int>(seq_lens), nseq, sk,
         (float)scale, (int)window, max_q, heads, rank, rot, block_size, nsplit,
-        nsplit > 1 ? ptr<float>(part_acc) : nullptr,
+        two_term ? 1 : 0, nsplit > 1 ? ptr<float>(part_acc) : nullptr,
         nsplit > 1 ? ptr<float>(part_ml) : nullptr, stream());
     return;
   }
@@ -139,22 +139,24 @@ void latent_attention_prefill(torch::Tensor out, torch::Tensor q_lat,
                               torch::Tensor block_tables, torch::Tensor qsl,
                               torch::Tensor seq_lens, double scale,
                               int64_t window, c10::optional<torch::Tensor> sinks,
-                              int64_t max_query_len, bool generic) {
+                              int64_t max_query_len, bool generic,
+                              bool two_term) {
   check_i32(qsl, "query_start_loc");
   TORCH_CHECK(qsl.numel() == seq_lens.numel() + 1);
   TORCH_CHECK(max_query_len >= 1, "max_query_len");
   latent_attention_common(out, q_lat, q_rot, cache, block_tables, ptr<int>(qsl),
                           seq_lens, scale, window, sinks, (int)max_query_len,
-                          !generic);
+                          !generic, two_term);
 }
 
 void latent_attention_decode(torch::Tensor out, torch::Tensor q_lat,
                              torch::Tensor q_rot, torch::Tensor cache,
                              torch::Tensor block_tables, torch::Tensor seq_lens,
                              double scale, int64_t window,
-                             c10::optional<torch::Tensor> sinks, bool generic) {
+                             c10::optional<torch::Tensor> sinks, bool generic,
+                             bool two_term) {
   latent_attention_common(out, q_lat, q_rot, cache, block_tables, nullptr,
-                          seq_lens, scale, window, sinks, 1, !generic);
+                          seq_lens, scale, window, sinks, 1, !generic, two_term);
 }
 
 }  // namespace

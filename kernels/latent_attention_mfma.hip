@@ -57,8 +57,8 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
     const bf16* __restrict__ cache, const int* __restrict__ block_tables,
     int bt_stride, const int* __restrict__ qsl, const int* __restrict__ seq_lens,
     const float* __restrict__ sinks, float scale, int window, int heads, int tq,
-    int hpb, int block_size, int nsplit, float* __restrict__ part_acc,
-    float* __restrict__ part_ml) {
+    int hpb, int block_size, int nsplit, int two_term,
+    float* __restrict__ part_acc, float* __restrict__ part_ml) {
   constexpr int RANK = NT * 16;
   constexpr int D = KS * 32;
   constexpr int KROW = D + LM_KPAD;
@@ -203,6 +203,9 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
     }
   };
   bf16x8_t pb;   // this tile's probabilities, B operand of the value product
+  // two_term: what rounding to bf16 left of them, a second B operand, so that
+  // the weights reach the value product with 16 mantissa bits
+  bf16x8_t pb_rest = {};
   auto scores = [&](const bf16* kb, int base) {
     f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
     if (wave_active) {
@@ -237,6 +240,9 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
       const float p = (sv[i] == -INFINITY) ? 0.f : __expf(sv[i] - m_safe);
       ps += p;
       pb[i] = f32_to_bf16_bits(p);
+      if (two_term)
+        pb_rest[i] = f32_to_bf16_bits(
+            p - __uint_as_float(((unsigned)(unsigned short)pb[i]) << 16));
     }
     l_part = l_part * alpha + ps;
     m_run = m_new;
@@ -252,6 +258,8 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
         const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(
             vb + ((dp * NTW + dt) * 16 + n) * LM_VROW + g * 8);
         acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, acc[dt], 0, 0, 0);
+        if (two_term)
+          acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb_rest, acc[dt], 0, 0, 0);
       }
     }
   };
@@ -399,7 +407,8 @@ static void launch_one(bf16* out, long o_st, long o_sh, const bf16* q_lat,
                        int bt_stride, const int* qsl, const int* seq_lens,
                        int nseq, const float* sinks, float scale, int window,
                        int max_q, int heads, int block_size, int nsplit,
-                       float* part_acc, float* part_ml, hipStream_t stream) {
+                       int two_term, float* part_acc, float* part_ml,
+                       hipStream_t stream) {
   constexpr int RANK = NT * 16, D = KS * 32;
   const size_t smem = sizeof(bf16) * (LM_KT * (D + LM_KPAD) + RANK * LM_VROW) *
                           1 +
@@ -417,7 +426,7 @@ static void launch_one(bf16* out, long o_st, long o_sh, const bf16* q_lat,
   latent_attn_mfma_kernel<NT, KS, DS><<<grid, LM_THREADS, smem, stream>>>(
       out, o_st, o_sh, q_lat, ql_st, ql_sh, q_rot, qr_st, qr_sh, cache,
       block_tables, bt_stride, qsl, seq_lens, sinks, scale, window, heads, tq,
-      hpb, block_size, nsplit, part_acc, part_ml);
+      hpb, block_size, nsplit, two_term, part_acc, part_ml);
   if (nsplit > 1) {
     dim3 mg(nseq, heads);
     latent_attn_merge_kernel<<<mg, 128, 0, stream>>>(out, o_st, o_sh, part_acc, part_ml,
@@ -432,8 +441,9 @@ void launch_latent_attn_mfma(bf16* out, long o_st, long o_sh, const bf16* q_lat,
                              const int* qsl, const int* seq_lens, int nseq,
                              const float* sinks, float scale, int window,
                              int max_q, int heads, int rank, int rot,
-                             int block_size, int nsplit, float* part_acc,
-                             float* part_ml, hipStream_t stream) {
+                             int block_size, int nsplit, int two_term,
+                             float* part_acc, float* part_ml,
+                             hipStream_t stream) {
   const int nt = rank / 16, ks = (rank + rot) / 32;
   // one query per sequence and at most one 16-row tile of heads
   // single queries: as many waves per row tile as the head count leaves free.
@@ -447,17 +457,20 @@ void launch_latent_attn_mfma(bf16* out, long o_st, long o_sh, const bf16* q_lat,
       launch_one<A, B, (A % 4 == 0 ? 4 : 1)>(                                 \
           out, o_st, o_sh, q_lat, ql_st, ql_sh, q_rot, qr_st, qr_sh, cache,  \
           block_tables, bt_stride, qsl, seq_lens, nseq, sinks, scale, window, \
-          max_q, heads, block_size, nsplit, part_acc, part_ml, stream);       \
+          max_q, heads, block_size, nsplit, two_term, part_acc, part_ml,      \
+          stream);                                                            \
     else if (dim_split >= 2)                                                  \
       launch_one<A, B, 2>(                                                    \
           out, o_st, o_sh, q_lat, ql_st, ql_sh, q_rot, qr_st, qr_sh, cache,  \
           block_tables, bt_stride, qsl, seq_lens, nseq, sinks, scale, window, \
-          max_q, heads, block_size, nsplit, part_acc, part_ml, stream);       \
+          max_q, heads, block_size, nsplit, two_term, part_acc, part_ml,      \
+          stream);                                                            \
     else                                                                      \
       launch_one<A, B, 1>(                                                    \
           out, o_st, o_sh, q_lat, ql_st, ql_sh, q_rot, qr_st, qr_sh, cache,  \
           block_tables, bt_stride, qsl, seq_lens, nseq, sinks, scale, window, \
-          max_q, heads, block_size, nsplit, part_acc, part_ml, stream);       \
+          max_q, heads, block_size, nsplit, two_term, part_acc, part_ml,      \
+          stream);                                                            \
     return;                                                                   \
   }
   LM_SHAPES(X)

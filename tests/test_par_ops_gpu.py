@@ -327,3 +327,41 @@ def test_window_edge_on_matrix_cores(dim, n_new, window):
         assert (float(want.abs().max()) > 50.0) == seen
         got = out[-1, 0].double().cpu()
         assert float((got - want).abs().max()) < 0.6, f"spike at {at}: {got[:3]} vs {want[:3]}"
+
+
+@pytest.mark.parametrize("two_term", [False, True])
+@pytest.mark.parametrize("rank,rot", [(64, 32), (256, 32)])
+def test_latent_attention_two_term_weights(rank, rot, two_term):
+    """The latent MFMA kernel with one or two bf16 terms per softmax weight
+    against the reference, portions and single queries."""
+    g = torch.Generator().manual_seed(10)
+    dtype, heads, bs = torch.bfloat16, 4, 16
+    spec = [(200, 200), (3, 150), (40, 333)]
+    ctxs = [s[1] for s in spec]
+    nb = sum((c + bs - 1) // bs for c in ctxs) + 2
+    cache = (torch.randn(nb, bs, rank + rot, generator=g) * 0.5).to(dtype)
+    perm = torch.randperm(nb, generator=g).tolist()
+    width = max((c + bs - 1) // bs for c in ctxs)
+    bt = torch.zeros(len(ctxs), width, dtype=torch.int32)
+    for i, c in enumerate(ctxs):
+        n = (c + bs - 1) // bs
+        bt[i, :n] = torch.tensor([perm.pop() for _ in range(n)], dtype=torch.int32)
+    news = [s[0] for s in spec]
+    qsl = torch.tensor([0] + torch.tensor(news).cumsum(0).tolist(), dtype=torch.int32)
+    lens = torch.tensor(ctxs, dtype=torch.int32)
+    t = int(qsl[-1])
+    ql = (torch.randn(t, heads, rank, generator=g) * 0.3).to(dtype)
+    qr = (torch.randn(t, heads, rot, generator=g) * 0.3).to(dtype)
+    want = ref.latent_attention(ql, qr, cache, bt, qsl, lens, 0.2, 0, None)
+    out = torch.empty(t, heads, rank, dtype=dtype, device=DEV)
+    ops.latent_attention_prefill(ql.to(DEV), qr.to(DEV), cache.to(DEV), bt.to(DEV), qsl.to(DEV),
+                                 lens.to(DEV), 0.2, 0, None, max(news), out=out,
+                                 two_term=two_term)
+    _close(out, want, dtype, "portions")
+    q1l, q1r = ql[:3].contiguous(), qr[:3].contiguous()
+    want1 = ref.latent_attention(q1l, q1r, cache, bt, torch.arange(4, dtype=torch.int32), lens,
+                                 0.2, 0, None)
+    out1 = torch.empty(3, heads, rank, dtype=dtype, device=DEV)
+    ops.latent_attention_decode(q1l.to(DEV), q1r.to(DEV), cache.to(DEV), bt.to(DEV),
+                                lens.to(DEV), 0.2, 0, None, out=out1, two_term=two_term)
+    _close(out1, want1, dtype, "single queries")

@@ -149,10 +149,13 @@ class LatentAttention(nn.Module):
                  rank: int, scale: float, window: int, rot_base: float,
                  rot_dims: int, eps: float, kv_owner: bool, has_sink: bool,
                  dtype: torch.dtype, rot_interleaved: bool = False,
-                 rot_scaling: Optional[dict] = None, head_gate: bool = False):
+                 rot_scaling: Optional[dict] = None, head_gate: bool = False,
+                 two_term_weights: bool = False):
         """``rot_interleaved``: dim 2i is paired with 2i+1 instead of i with
         i + rot_dims/2.  ``rot_scaling``: see ``scaled_rotary_frequencies``.
-        ``head_gate``: head h's output is multiplied by sigmoid(W_g x)_h."""
+        ``head_gate``: head h's output is multiplied by sigmoid(W_g x)_h.
+        ``two_term_weights``: the bf16 matrix-core kernel feeds the softmax
+        weights to the value product as two bf16 terms (16 mantissa bits)."""
         super().__init__()
         tp = get_tp_world_size()
         self.heads = divide(heads, tp)
@@ -181,6 +184,7 @@ class LatentAttention(nn.Module):
             requires_grad=False)
         self.sink = _f32_param(self.heads) if has_sink else None
         self.rot_interleaved = rot_interleaved
+        self.two_term_weights = two_term_weights
         freqs, self.rot_mag = scaled_rotary_frequencies(rot_base, rot_dims, rot_scaling)
         self.register_buffer(
             "inv_freq", torch.tensor(freqs, dtype=torch.float64).to(torch.float32),
@@ -238,12 +242,12 @@ class LatentAttention(nn.Module):
                 q_lat[:npt], q_rot[:npt], cache, meta.prefill_block_tables,
                 meta.prefill_query_start_loc, meta.prefill_seq_lens, self.scale,
                 self.window, self.sink, meta.max_prefill_query_len,
-                out=o_view[:npt])
+                out=o_view[:npt], two_term=self.two_term_weights)
         if meta.num_decode_seqs:
             ops.latent_attention_decode(
                 q_lat[npt:], q_rot[npt:], cache, meta.decode_block_tables,
                 meta.decode_seq_lens, self.scale, self.window, self.sink,
-                out=o_view[npt:])
+                out=o_view[npt:], two_term=self.two_term_weights)
         o = torch.bmm(o_lat, self.uv_t)                    # [H, T, vdim]
         if self.head_gate:
             # gate and the [H, T] -> [T, H] regrouping in one pass

@@ -85,7 +85,7 @@ def build_mixer(kind: str, m: dict, width: int, eps: float, dtype: torch.dtype):
             vdim=int(m["vdim"]), rank=int(m["kv_rank"]), scale=float(m["scale"]),
             window=0, rot_base=float(rot.get("base", 10000.0)), rot_dims=rot_dim,
             eps=eps, kv_owner=True, has_sink=False, dtype=dtype, rot_interleaved=True,
-            rot_scaling=rot.get("scaling"), head_gate=True)
+            rot_scaling=rot.get("scaling"), head_gate=True, two_term_weights=True)
     raise ValueError(f"unknown mixer type {kind!r}")
 
 

@@ -641,15 +641,19 @@ def latent_kv_write(dkv, norm_weight, eps, positions, inv_freq, rot_dims,
 
 def latent_attention_prefill(q_lat, q_rot, cache, block_tables, query_start_loc,
                              seq_lens, scale, window, sinks, max_query_len,
-                             out: torch.Tensor, general: bool = False) -> torch.Tensor:
+                             out: torch.Tensor, general: bool = False,
+                             two_term: bool = False) -> torch.Tensor:
     """Windowed multi-query attention with sinks over the paged latent cache
     for query chunks (the tail rows of each sequence).  bf16 shapes on the
     MFMA kernel's list run there unless ``general`` asks for the any-shape
-    kernel (f32 always does)."""
+    kernel (f32 always does).  ``two_term``: on the MFMA kernel the
+    probabilities enter the value product as two bf16 terms (rounded value +
+    rounded remainder) instead of one."""
     if q_lat.numel() and _native_lat(q_lat):
         _L.latent_attention_prefill(out, q_lat, q_rot, cache, block_tables,
                                     query_start_loc, seq_lens, float(scale),
-                                    int(window), sinks, int(max_query_len), bool(general))
+                                    int(window), sinks, int(max_query_len), bool(general),
+                                    bool(two_term))
         return out
     out.copy_(reference.latent_attention(
         q_lat, q_rot, cache, block_tables.cpu(), query_start_loc.cpu(),
@@ -659,12 +663,12 @@ def latent_attention_prefill(q_lat, q_rot, cache, block_tables, query_start_loc,
 
 def latent_attention_decode(q_lat, q_rot, cache, block_tables, seq_lens, scale,
                             window, sinks, out: torch.Tensor,
-                            general: bool = False) -> torch.Tensor:
+                            general: bool = False, two_term: bool = False) -> torch.Tensor:
     """Same attention for one new query per sequence."""
     if q_lat.numel() and _native_lat(q_lat):
         _L.latent_attention_decode(out, q_lat, q_rot, cache, block_tables,
                                    seq_lens, float(scale), int(window), sinks,
-                                   bool(general))
+                                   bool(general), bool(two_term))
         return out
     n = q_lat.shape[0]
     qsl = torch.arange(n + 1, dtype=torch.int32)
