@@ -135,9 +135,11 @@ def dense_ff(h, w_up, b_up, w_down, b_down):
     return relu_squared(h @ w_up.T + b_up) @ w_down.T + b_down
 
 
-def routed_ff(h, w_router, correction, experts, *, top, identity):
+def routed_ff(h, w_router, correction, experts, *, top, identity, margins=None):
     """experts: list of (w_up, w_down); the last ``identity`` router outputs
-    are experts that return their input."""
+    are experts that return their input.  ``margins`` (a list) receives, per
+    token, the gap between the last chosen and the first unchosen choice
+    score: a small gap is a close call that rounding may decide otherwise."""
     n = h.shape[0]
     z = h @ w_router.T
     s = torch.softmax(z, dim=-1)
@@ -145,7 +147,11 @@ def routed_ff(h, w_router, correction, experts, *, top, identity):
     out = torch.zeros_like(h)
     real = len(experts)
     for t in range(n):
-        order = sorted(range(real + identity), key=lambda e: (-float(choice[t, e]), e))[:top]
+        ranked = sorted(range(real + identity), key=lambda e: (-float(choice[t, e]), e))
+        order = ranked[:top]
+        if margins is not None:
+            margins.append(float(choice[t, ranked[top - 1]] - choice[t, ranked[top]])
+                           if top < real + identity else float("inf"))
         tot = sum(float(s[t, e]) for e in order) + 1e-20
         for e in order:
             wgt = float(s[t, e]) / tot
@@ -159,8 +165,10 @@ def routed_ff(h, w_router, correction, experts, *, top, identity):
 
 # -- the model --------------------------------------------------------------
 
-def forward(cfg: dict, w: dict, tokens: list[int], layers_out: list | None = None):
-    """Logits [n, vocab] of one whole sequence."""
+def forward(cfg: dict, w: dict, tokens: list[int], layers_out: list | None = None,
+            margins_out: list | None = None):
+    """Logits [n, vocab] of one whole sequence.  ``margins_out`` receives one
+    list per routed layer with every token's router margin (see routed_ff)."""
     w = {k: v.to(F64) for k, v in w.items()}
     eps = float(cfg["norm"]["eps"])
     x = w["embed"][torch.tensor(tokens)]
@@ -194,8 +202,12 @@ def forward(cfg: dict, w: dict, tokens: list[int], layers_out: list | None = Non
                 r = mlp["router"]
                 experts = [(w[f"{p}mlp.e{e}.up"], w[f"{p}mlp.e{e}.down"])
                            for e in range(int(r["experts"]))]
+                m_list = [] if margins_out is not None else None
                 y = y + routed_ff(h2, w[p + "mlp.router"], w[p + "mlp.correction"], experts,
-                                  top=int(r["top"]), identity=int(r.get("identity", 0)))
+                                  top=int(r["top"]), identity=int(r.get("identity", 0)),
+                                  margins=m_list)
+                if margins_out is not None:
+                    margins_out.append(m_list)
         x = x + y
         if layers_out is not None:
             layers_out.append(x.clone())

@@ -404,18 +404,26 @@ def test_bf16_stays_near_oracle(model, device):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_matrix_core_shapes(tmp_path, dtype):
     """Head sizes the matrix-core attention kernels take, long enough for
-    several key tiles, windows that end inside a tile."""
+    several key tiles, windows that end inside a tile; experts of a size the
+    grouped product takes (bf16 runs them grouped, f32 stacked)."""
     layers = [("attention", attn_spec(4, 2, 64, window=70, rot_dims=32), dense(64)),
-              ("latent_attention", latent_spec(4, 32, 32, 48, 64), moe(3, 1, 2, 16)),
+              ("latent_attention", latent_spec(4, 32, 32, 48, 64), moe(5, 1, 2, 128)),
               ("attention", attn_spec(8, 1, 128, window=33, rot_dims=128), None)]
-    cfg = make_config(layers, width=64, vocab=40)
+    cfg = make_config(layers, width=128, vocab=40)
     w = oracle.random_weights(cfg, seed=8)
     oracle.write_model(str(tmp_path / "m"), cfg, w)
     toks = _tokens(150, cfg["vocab"], 9)
-    want = oracle.forward(cfg, w, toks)
+    margins = []
+    want = oracle.forward(cfg, w, toks, margins_out=margins)
+    # a router's close call may go the other way in bf16: those positions prove
+    # nothing (what later positions see of them stays within the tolerance)
+    keep = [t for t in range(len(toks))
+            if dtype == "float32" or min(m[t] for m in margins) > 1e-3]
+    assert len(keep) > len(toks) - 10
     eng = _engine(str(tmp_path / "m"), "cuda", dtype=dtype, blocks=40, block_size=16)
-    _close(_feed(eng, "a", toks, [150]), want, dtype, "whole")
-    _close(_feed(eng, "b", toks, [70, 3, 40, 2] + [1] * 35), want, dtype, "portions")
+    assert eng.worker.model.layers[1].mlp.grouped == (dtype == "bfloat16")
+    _close(_feed(eng, "a", toks, [150])[keep], want[keep], dtype, "whole")
+    _close(_feed(eng, "b", toks, [70, 3, 40, 2] + [1] * 35)[keep], want[keep], dtype, "portions")
 
 
 @pytest.mark.gpu
