@@ -24,14 +24,14 @@ void launch_relu2(T*, const T*, long, const T*, const float*, int, int, int,
                   hipStream_t);
 int moe_route_max_experts();
 void launch_moe_route(float*, float*, int*, float*, const float*, const float*,
-                      int, int, int, int, hipStream_t);
+                      int, int, int, int, int, hipStream_t);
 template <typename T>
 void launch_moe_combine(T*, const T*, const int*, const int*, const float*, int,
                         int, int, int, hipStream_t);
 int moe_sort_max_experts();
 template <typename T>
 void launch_moe_sort(T*, int*, int*, int*, const T*, long, const int*, int, int,
-                     int, int, hipStream_t);
+                     int, int, const float*, hipStream_t);
 void launch_moe_gemm(__hip_bfloat16*, const __hip_bfloat16*,
                      const __hip_bfloat16*, const int*, int, int, int, int, int,
                      hipStream_t);
@@ -238,7 +238,25 @@ void moe_route(torch::Tensor dense, torch::Tensor ident, torch::Tensor ids,
   if (tokens == 0) return;
   launch_moe_route(ptr<float>(dense), ptr<float>(ident), ptr<int>(ids), ptr<float>(wts),
                    ptr<float>(logits), ptr<float>(correction), tokens, n, (int)num_real,
-                   top, stream());
+                   top, 0, stream());
+}
+
+// sigmoid scores, the top ones as they are (no correction, no renormalising)
+void moe_route_sigmoid(torch::Tensor dense, torch::Tensor ids, torch::Tensor wts,
+                       torch::Tensor logits) {
+  check_f32(logits, "logits");
+  check_f32(dense, "dense");
+  check_f32(wts, "weights");
+  check_i32(ids, "ids");
+  TORCH_CHECK(logits.dim() == 2 && ids.dim() == 2);
+  const int tokens = logits.size(0), n = logits.size(1), top = ids.size(1);
+  TORCH_CHECK(n <= moe_route_max_experts(), "too many router outputs");
+  TORCH_CHECK(top >= 1 && top <= n && ids.size(0) == tokens && wts.dim() == 2 &&
+              wts.size(0) == tokens && wts.size(1) == top &&
+              dense.numel() == (long)tokens * n);
+  if (tokens == 0) return;
+  launch_moe_route(ptr<float>(dense), nullptr, ptr<int>(ids), ptr<float>(wts),
+                   ptr<float>(logits), nullptr, tokens, n, n, top, 1, stream());
 }
 
 void moe_combine(torch::Tensor out, torch::Tensor ye, torch::Tensor pos,
@@ -262,7 +280,7 @@ void moe_combine(torch::Tensor out, torch::Tensor ye, torch::Tensor pos,
 
 void moe_sort(torch::Tensor xs, torch::Tensor pos, torch::Tensor seg,
               torch::Tensor scratch, torch::Tensor h, torch::Tensor ids,
-              int64_t num_real) {
+              int64_t num_real, c10::optional<torch::Tensor> row_scale) {
   check_i32(ids, "ids");
   check_i32(pos, "pos");
   check_i32(seg, "seg");
@@ -275,11 +293,16 @@ void moe_sort(torch::Tensor xs, torch::Tensor pos, torch::Tensor seg,
               scratch.numel() == 2 * num_real);
   TORCH_CHECK(xs.is_contiguous() && xs.dim() == 2 && xs.size(0) == (long)tokens * top &&
               xs.size(1) == width && xs.scalar_type() == h.scalar_type());
+  if (row_scale.has_value()) {
+    check_f32(row_scale.value(), "row_scale");
+    TORCH_CHECK(row_scale.value().sizes() == ids.sizes(), "row_scale is [tokens, top]");
+  }
   if (tokens == 0) return;
   DISPATCH_F32_BF16(h.scalar_type(), {
     launch_moe_sort<scalar_t>(ptr<scalar_t>(xs), ptr<int>(pos), ptr<int>(seg),
                               ptr<int>(scratch), ptr<scalar_t>(h), (long)h.stride(0),
-                              ptr<int>(ids), tokens, top, (int)num_real, width, stream());
+                              ptr<int>(ids), tokens, top, (int)num_real, width,
+                              optr<float>(row_scale), stream());
   });
 }
 
@@ -314,6 +337,7 @@ void register_par_ops(pybind11::module& m) {
   m.def("sigmoid_gate_mul", &sigmoid_gate_mul);
   m.def("relu2", &relu2);
   m.def("moe_route", &moe_route);
+  m.def("moe_route_sigmoid", &moe_route_sigmoid);
   m.def("moe_combine", &moe_combine);
   m.def("moe_sort", &moe_sort);
   m.def("moe_gemm", &moe_gemm);

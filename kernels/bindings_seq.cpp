@@ -21,7 +21,7 @@ void launch_stream_add(float*, const T*, const T*, float, T*, long, hipStream_t)
 template <typename T>
 void launch_stream_add_rms_norm(float*, const T*, const float*, float, float,
                                 int, int, T*, const float*, float, float,
-                                hipStream_t);
+                                const float*, hipStream_t);
 template <typename T>
 void launch_softcap(float*, const T*, float, long, hipStream_t);
 template <typename T>
@@ -41,6 +41,7 @@ void register_rec_ops(pybind11::module& m);
 // two-norm residual kernel, rotation + cache write, gates, squared relu,
 // expert router and combine (bindings_par.cpp)
 void register_par_ops(pybind11::module& m);
+void register_mix_ops(pybind11::module& m);
 namespace {
 
 hipStream_t stream() { return at::hip::getCurrentHIPStream().stream(); }
@@ -155,18 +156,26 @@ void stream_add_rms_norm(torch::Tensor x, torch::Tensor y, torch::Tensor weight,
                          double eps, double mult,
                          c10::optional<torch::Tensor> next_out,
                          c10::optional<torch::Tensor> next_weight,
-                         double next_eps, double next_offset) {
+                         double next_eps, double next_offset,
+                         c10::optional<torch::Tensor> layer_scale) {
+  // next_out without next_weight: the updated stream rounded to y's type
   check_f32(x, "x");
   check_f32(weight, "weight");
   const int width = x.size(-1);
   TORCH_CHECK(y.is_cuda() && y.is_contiguous() && y.numel() == x.numel() &&
               weight.numel() == width);
   const int rows = x.numel() / width;
-  TORCH_CHECK(next_out.has_value() == next_weight.has_value());
-  if (next_out.has_value()) {
+  TORCH_CHECK(next_out.has_value() || !next_weight.has_value());
+  if (layer_scale.has_value()) {
+    check_f32(layer_scale.value(), "layer_scale");
+    TORCH_CHECK(layer_scale.value().numel() == width);
+  }
+  if (next_weight.has_value()) {
     check_f32(next_weight.value(), "next_weight");
-    TORCH_CHECK(next_weight.value().numel() == width &&
-                next_out.value().is_contiguous() &&
+    TORCH_CHECK(next_weight.value().numel() == width);
+  }
+  if (next_out.has_value()) {
+    TORCH_CHECK(next_out.value().is_cuda() && next_out.value().is_contiguous() &&
                 next_out.value().numel() == x.numel() &&
                 next_out.value().scalar_type() == y.scalar_type());
   }
@@ -175,8 +184,9 @@ void stream_add_rms_norm(torch::Tensor x, torch::Tensor y, torch::Tensor weight,
         ptr<float>(x), ptr<scalar_t>(y), ptr<float>(weight), (float)eps,
         (float)mult, rows, width,
         next_out.has_value() ? ptr<scalar_t>(next_out.value()) : nullptr,
-        next_out.has_value() ? ptr<float>(next_weight.value()) : nullptr,
-        (float)next_eps, (float)next_offset, stream());
+        next_weight.has_value() ? ptr<float>(next_weight.value()) : nullptr,
+        (float)next_eps, (float)next_offset,
+        layer_scale.has_value() ? ptr<float>(layer_scale.value()) : nullptr, stream());
   });
 }
 

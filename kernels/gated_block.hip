@@ -347,7 +347,9 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
     float* __restrict__ dense, float* __restrict__ ident, int* __restrict__ ids,
     float* __restrict__ wts, const float* __restrict__ logits,
     const float* __restrict__ correction, int tokens, int n, int num_real,
-    int top) {
+    int top, int sigmoid) {
+  // sigmoid: scores are sigmoid(logit) instead of the softmax, there is no
+  // correction (nullptr), no identity output and no renormalising
   const int lane = threadIdx.x & (WAVE_SIZE - 1);
   const long t = blockIdx.x * (long)(blockDim.x / WAVE_SIZE) + threadIdx.x / WAVE_SIZE;
   if (t >= tokens) return;
@@ -362,20 +364,29 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
     taken[i] = false;
     m = fmaxf(m, s[i]);
   }
-  m = wave_reduce_max(m);
-  float den = 0.f;
+  if (sigmoid) {
 #pragma unroll
-  for (int i = 0; i < RT_MAX; ++i) {
-    const int e = lane + i * WAVE_SIZE;
-    s[i] = (e < n) ? expf(s[i] - m) : 0.f;
-    den += s[i];
-  }
-  den = wave_reduce_sum(den);
+    for (int i = 0; i < RT_MAX; ++i) {
+      const int e = lane + i * WAVE_SIZE;
+      s[i] = (e < n) ? 1.0f / (1.0f + expf(-s[i])) : 0.f;
+      ch[i] = (e < n) ? s[i] : -INFINITY;
+    }
+  } else {
+    m = wave_reduce_max(m);
+    float den = 0.f;
 #pragma unroll
-  for (int i = 0; i < RT_MAX; ++i) {
-    const int e = lane + i * WAVE_SIZE;
-    s[i] = s[i] / den;
-    ch[i] = (e < n) ? s[i] + correction[e] : -INFINITY;
+    for (int i = 0; i < RT_MAX; ++i) {
+      const int e = lane + i * WAVE_SIZE;
+      s[i] = (e < n) ? expf(s[i] - m) : 0.f;
+      den += s[i];
+    }
+    den = wave_reduce_sum(den);
+#pragma unroll
+    for (int i = 0; i < RT_MAX; ++i) {
+      const int e = lane + i * WAVE_SIZE;
+      s[i] = s[i] / den;
+      ch[i] = (e < n) ? s[i] + correction[e] : -INFINITY;
+    }
   }
   float total = 0.f, id_sum = 0.f;
   for (int k = 0; k < top; ++k) {
@@ -416,14 +427,14 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
       wts[t * top + k] = sv;
     }
   }
-  const float inv = 1.0f / (total + 1e-20f);
+  const float inv = sigmoid ? 1.0f : 1.0f / (total + 1e-20f);
 #pragma unroll
   for (int i = 0; i < RT_MAX; ++i) {
     const int e = lane + i * WAVE_SIZE;
     if (e < num_real) dense[t * num_real + e] = taken[i] ? s[i] * inv : 0.f;
   }
   // lane 0 wrote wts[t, :] itself, so it may rescale them in place
-  if (lane == 0) {
+  if (lane == 0 && !sigmoid) {
     for (int k = 0; k < top; ++k) wts[t * top + k] *= inv;
     ident[t] = id_sum * inv;
   }
@@ -523,22 +534,37 @@ template <typename T>
 __global__ __launch_bounds__(256) void moe_gather_kernel(
     T* __restrict__ xs, const T* __restrict__ h, long h_st,
     const int* __restrict__ pos, const int* __restrict__ ids, int top,
-    int num_real, int width, int vec) {
+    int num_real, int width, int vec, const float* __restrict__ row_scale) {
   const long t = blockIdx.x;
   const T* src = h + t * h_st;
   if (vec) {
     constexpr int V = Vec16<T>::kElems;
     for (int c = threadIdx.x * V; c < width; c += blockDim.x * V) {
       const Vec16<T> v = load16(src + c);
-      for (int k = 0; k < top; ++k)
-        if (ids[t * top + k] < num_real)
+      for (int k = 0; k < top; ++k) {
+        if (ids[t * top + k] >= num_real) continue;
+        if (row_scale == nullptr) {
           store16(xs + (long)pos[t * top + k] * width + c, v);
+        } else {
+          const float sc = row_scale[t * top + k];
+          Vec16<T> o;
+#pragma unroll
+          for (int u = 0; u < V; ++u)
+            o.data[u] = ScalarOps<T>::from_f32(ScalarOps<T>::to_f32(v.data[u]) * sc);
+          store16(xs + (long)pos[t * top + k] * width + c, o);
+        }
+      }
     }
   } else {
     for (int c = threadIdx.x; c < width; c += blockDim.x) {
       const T v = src[c];
-      for (int k = 0; k < top; ++k)
-        if (ids[t * top + k] < num_real) xs[(long)pos[t * top + k] * width + c] = v;
+      for (int k = 0; k < top; ++k) {
+        if (ids[t * top + k] >= num_real) continue;
+        xs[(long)pos[t * top + k] * width + c] =
+            row_scale == nullptr
+                ? v
+                : ScalarOps<T>::from_f32(ScalarOps<T>::to_f32(v) * row_scale[t * top + k]);
+      }
     }
   }
 }
@@ -555,7 +581,7 @@ int moe_sort_max_experts() { return MS_MAX; }
 template <typename T>
 void launch_moe_sort(T* xs, int* pos, int* seg, int* counts_cursor, const T* h,
                      long h_st, const int* ids, int tokens, int top, int num_real,
-                     int width, hipStream_t s) {
+                     int width, const float* row_scale, hipStream_t s) {
   const int npairs = tokens * top;
   const int blocks = grid_for(npairs, 256) > 1024 ? 1024 : grid_for(npairs, 256);
   moe_count_kernel<<<blocks, 256, 0, s>>>(counts_cursor, ids, npairs, num_real);
@@ -564,7 +590,7 @@ void launch_moe_sort(T* xs, int* pos, int* seg, int* counts_cursor, const T* h,
   constexpr int V = Vec16<T>::kElems;
   const int vec = width % V == 0 && h_st % V == 0 && al(xs, 16) && al(h, 16);
   moe_gather_kernel<T><<<tokens, 256, 0, s>>>(xs, h, h_st, pos, ids, top, num_real,
-                                             width, vec);
+                                             width, vec, row_scale);
 }
 
 template <typename T>
@@ -652,10 +678,10 @@ int moe_route_max_experts() { return RT_MAX * WAVE_SIZE; }
 
 void launch_moe_route(float* dense, float* ident, int* ids, float* wts,
                       const float* logits, const float* correction, int tokens,
-                      int n, int num_real, int top, hipStream_t s) {
+                      int n, int num_real, int top, int sigmoid, hipStream_t s) {
   const int waves = 256 / WAVE_SIZE;
   moe_route_kernel<<<(tokens + waves - 1) / waves, 256, 0, s>>>(
-      dense, ident, ids, wts, logits, correction, tokens, n, num_real, top);
+      dense, ident, ids, wts, logits, correction, tokens, n, num_real, top, sigmoid);
 }
 
 template <typename T>
@@ -672,7 +698,8 @@ void launch_moe_combine(T* out, const T* ye, const int* pos, const int* ids,
 
 #define INSTANTIATE(T)                                                           \
   template void launch_moe_sort<T>(T*, int*, int*, int*, const T*, long,         \
-                                   const int*, int, int, int, int, hipStream_t); \
+                                   const int*, int, int, int, int, const float*, \
+                                   hipStream_t);                                 \
   template void launch_stream_add_rms_norm_pair<T>(                              \
       float*, const T*, const T*, const float*, const T*, const float*,          \
       const float*, float, int, int, T*, T*, hipStream_t);                       \

@@ -161,7 +161,10 @@ __global__ void stream_add_rms_norm_kernel(float* __restrict__ x,
                                            float eps, float mult, int width,
                                            T* __restrict__ next_out,
                                            const float* __restrict__ next_w,
-                                           float next_eps, float next_offset) {
+                                           float next_eps, float next_offset,
+                                           const float* __restrict__ ls) {
+  // ls: optional per-channel layer scale on the normed rows.  next_out without
+  // next_w: the updated stream rounded to T, no norm.
   const long row = blockIdx.x;
   const T* yr = y + row * width;
   float* xr = x + row * width;
@@ -185,16 +188,27 @@ __global__ void stream_add_rms_norm_kernel(float* __restrict__ x,
       const F4 f = Pack4<T>::load(yr + c);
       const F4 g = Pack4<float>::load(w + c);
       F4 v = Pack4<float>::load(xr + c);
+      if (ls != nullptr) {
+        const F4 l = Pack4<float>::load(ls + c);
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        v.v[k] += mult * (f.v[k] * inv * g.v[k]);
-        sx += v.v[k] * v.v[k];
+        for (int k = 0; k < 4; ++k) v.v[k] += mult * (f.v[k] * inv * g.v[k] * l.v[k]);
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v.v[k] += mult * (f.v[k] * inv * g.v[k]);
       }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) sx += v.v[k] * v.v[k];
       Pack4<float>::store(xr + c, v);
+      if (next_out != nullptr && next_w == nullptr)
+        Pack4<T>::store(next_out + row * width + c, v);
     } else {
-      const float v = xr[c] + mult * (ScalarOps<T>::to_f32(yr[c]) * inv * w[c]);
+      float n = ScalarOps<T>::to_f32(yr[c]) * inv * w[c];
+      if (ls != nullptr) n *= ls[c];
+      const float v = xr[c] + mult * n;
       xr[c] = v;
       sx += v * v;
+      if (next_out != nullptr && next_w == nullptr)
+        next_out[row * width + c] = ScalarOps<T>::from_f32(v);
     }
   }
   if (next_w == nullptr) return;
@@ -354,14 +368,14 @@ template <typename T>
 void launch_stream_add_rms_norm(float* x, const T* y, const float* w, float eps,
                                 float mult, int rows, int width, T* next_out,
                                 const float* next_w, float next_eps,
-                                float next_offset, hipStream_t s) {
+                                float next_offset, const float* ls, hipStream_t s) {
   if (width % 4 == 0 && al(x, 16) && al(y, 4 * sizeof(T)) && al(w, 16) &&
-      al(next_out, 4 * sizeof(T)) && al(next_w, 16))
+      al(next_out, 4 * sizeof(T)) && al(next_w, 16) && al(ls, 16))
     stream_add_rms_norm_kernel<T, true><<<rows, 256, 0, s>>>(
-        x, y, w, eps, mult, width, next_out, next_w, next_eps, next_offset);
+        x, y, w, eps, mult, width, next_out, next_w, next_eps, next_offset, ls);
   else
     stream_add_rms_norm_kernel<T, false><<<rows, 256, 0, s>>>(
-        x, y, w, eps, mult, width, next_out, next_w, next_eps, next_offset);
+        x, y, w, eps, mult, width, next_out, next_w, next_eps, next_offset, ls);
 }
 template <typename T>
 void launch_softcap(float* out, const T* in, float cap, long n, hipStream_t s) {
@@ -398,7 +412,7 @@ void launch_latent_kv_write(const T* dkv, const float* norm_w, float eps,
   template void launch_stream_add_rms_norm<T>(float*, const T*, const float*,   \
                                               float, float, int, int, T*,       \
                                               const float*, float, float,       \
-                                              hipStream_t);                     \
+                                              const float*, hipStream_t);       \
   template void launch_softcap<T>(float*, const T*, float, long, hipStream_t);  \
   template void launch_rope_partial<T>(T*, long, long, const long*,             \
                                        const float*, int, int, int, int, int,   \

@@ -167,6 +167,10 @@ def _from_hf_config(model: str, hf: dict) -> ModelConfig:
         from ..models.relerax import model_config_from_json
 
         return model_config_from_json(model, hf)
+    if hf.get("architecture") == "Gumozen":
+        from ..models.gumozen import model_config_from_json
+
+        return model_config_from_json(model, hf)
     arch_list = hf.get("architectures") or []
     arch = "llama"
     if any("Mixtral" in a for a in arch_list):

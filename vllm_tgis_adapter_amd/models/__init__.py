@@ -30,6 +30,10 @@ def get_model(cfg: ModelConfig):
         from .relerax import ReleraxForCausalLM
 
         return ReleraxForCausalLM(cfg)
+    if cfg.architecture == "gumozen":
+        from .gumozen import GumozenForCausalLM
+
+        return GumozenForCausalLM(cfg)
     raise ValueError(f"Unsupported architecture: {cfg.architecture}")
 
 
@@ -47,4 +51,8 @@ def native_extensions(cfg: ModelConfig) -> list[str]:
         from .relerax import native_extensions as rx
 
         return rx(cfg)
+    if cfg.architecture == "gumozen":
+        from .gumozen import native_extensions as gz
+
+        return gz(cfg)
     return ["_C"]

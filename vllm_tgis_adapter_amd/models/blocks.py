@@ -35,6 +35,19 @@ that another design can assemble them differently:
 - ``BiasedDenseMLP``    down(act(up h + b) ) + b with a squared relu
 - ``RoutedExperts``     softmax router with a choice correction, top-k of
                         small squared-relu experts plus identity experts
+- ``TokenShift``        per-channel blend of a row of the f32 stream with the
+                        row before it, the last row carried per sequence
+- ``DiffAttention``     differential grouped-query attention: two softmax maps
+                        over the same values, query/key norm, rotation with
+                        piecewise frequency scaling, a chunk mask, a per-head
+                        sigmoid gate
+- ``HGRN2Mixer``        gated linear recurrence whose forget gate (with a
+                        per-channel lower bound) also sets what is written
+- ``GatedRoutedExperts`` sigmoid router, top-k of small gated (silu) experts
+                        whose input is multiplied by the routing weight
+- ``stepped_rotary_frequencies``  rotation frequencies divided by a factor
+                        for long wavelengths, kept for short ones, blended
+                        linearly in between
 
 The recurrent mixers keep their state (f32) and the last inputs of their short
 convolutions in per-sequence slots; a sequence that starts in a step starts
@@ -150,8 +163,10 @@ class LatentAttention(nn.Module):
                  rot_dims: int, eps: float, kv_owner: bool, has_sink: bool,
                  dtype: torch.dtype, rot_interleaved: bool = False,
                  rot_scaling: Optional[dict] = None, head_gate: bool = False,
-                 two_term_weights: bool = False):
-        """``rot_interleaved``: dim 2i is paired with 2i+1 instead of i with
+                 two_term_weights: bool = False, q_rank: int = 0):
+        """``q_rank`` > 0: queries go through a latent of that size, q = W_uq
+        rmsnorm(W_dq h) (plain weight, eps of the layer).
+        ``rot_interleaved``: dim 2i is paired with 2i+1 instead of i with
         i + rot_dims/2.  ``rot_scaling``: see ``scaled_rotary_frequencies``.
         ``head_gate``: head h's output is multiplied by sigmoid(W_g x)_h.
         ``two_term_weights``: the bf16 matrix-core kernel feeds the softmax
@@ -164,7 +179,13 @@ class LatentAttention(nn.Module):
         self.rot_dims = rot_dims
         self.kv_owner = kv_owner
         self.dtype = dtype
-        self.q_proj = ColumnParallelLinear(width, heads * (dim + rot_dim), dtype=dtype)
+        self.q_rank = q_rank
+        self.q_proj = ColumnParallelLinear(q_rank or width, heads * (dim + rot_dim), dtype=dtype)
+        if q_rank:
+            # replicated on every rank, like the key/value latent
+            self.dq_weight = nn.Parameter(
+                torch.empty(q_rank, width, dtype=dtype).normal_(0.0, 0.02), requires_grad=False)
+            self.dq_norm = _f32_param(q_rank, fill=1.0)
         self.o_proj = RowParallelLinear(heads * vdim, width, dtype=dtype)
         if kv_owner:
             # replicated on every rank: the latent is shared by all heads.  With a
@@ -196,9 +217,13 @@ class LatentAttention(nn.Module):
                          requires_grad=False) if head_gate and not kv_owner else None)
 
     # -- weights -----------------------------------------------------------
-    def load(self, q, dkv, dkv_norm, uk, uv, sink, o, gate=None) -> None:
+    def load(self, q, dkv, dkv_norm, uk, uv, sink, o, gate=None, dq=None,
+             dq_norm=None) -> None:
         r, h = get_tp_rank(), self.heads
         self.q_proj.load_full_weight(q)
+        if self.q_rank:
+            self.dq_weight.data.copy_(dq.to(self.dtype))
+            self.dq_norm.data.copy_(dq_norm.float())
         self.o_proj.load_full_weight(o)
         if self.gate_weight is not None:
             self.gate_weight.data.copy_(gate[r * h:(r + 1) * h].to(self.dtype))
@@ -220,9 +245,15 @@ class LatentAttention(nn.Module):
                 cache: torch.Tensor, meta: AttnMetadata) -> torch.Tensor:
         t = h.shape[0]
         nh, d, r, rank = self.heads, self.dim, self.rot_dim, self.rank
-        q = self.q_proj(h).view(t, nh, d + r)
-        ops.rope_partial(q, positions, self.inv_freq, d, self.rot_dims,
-                         self.rot_interleaved, self.rot_mag)
+        if self.q_rank:
+            cq = ops.group_rms_norm(ops.linear(h, self.dq_weight), self.dq_norm, 1,
+                                    self.eps, self.dtype)
+            q = self.q_proj(cq).view(t, nh, d + r)
+        else:
+            q = self.q_proj(h).view(t, nh, d + r)
+        if self.rot_dims:
+            ops.rope_partial(q, positions, self.inv_freq, d, self.rot_dims,
+                             self.rot_interleaved, self.rot_mag)
         g = None
         if self.kv_owner:
             dkv = ops.linear(h, self.dkv_weight)
@@ -842,3 +873,261 @@ class RoutedExperts(nn.Module):
         a = ops.moe_gemm(xs, self.up, seg, gated=False, act="relu2")
         ye = ops.moe_gemm(a, self.down, seg, gated=False)
         return ops.moe_combine(ye, pos, ids, w, ne), ident
+
+
+# ---------------------------------------------------------------------------
+# Token shift, differential attention with a chunk mask, HGRN2, sigmoid-routed
+# gated experts.
+# ---------------------------------------------------------------------------
+
+
+class TokenShift(nn.Module):
+    """h_t + (h_(t-1) - h_t) * w per channel, h the f32 stream as it is before
+    the blend; the row before position 0 is zero.  The last row of every
+    portion is kept per sequence (f32 [width]) so that portions of any size
+    continue where the previous one ended."""
+
+    def __init__(self, width: int, dtype: torch.dtype):
+        super().__init__()
+        self.width, self.dtype = width, dtype
+        self.weight = _f32_param(width)
+
+    def state_shape(self) -> tuple:
+        return ("slot", (self.width,), torch.float32)
+
+    def forward(self, x: torch.Tensor, state: torch.Tensor, meta: AttnMetadata) -> torch.Tensor:
+        return ops.token_shift_state(x, self.weight, state, meta.seq_start_loc,
+                                     meta.seq_lens, meta.state_slots, self.dtype)
+
+
+def stepped_rotary_frequencies(base: float, dims: int,
+                               scaling: Optional[dict] = None) -> list:
+    """Frequencies of the dims/2 rotated pairs, f_i = base^(-2i/dims).
+
+    ``scaling`` = {factor, low, high, original}: with the wavelength l = 2 pi /
+    f, pairs with l < original/high keep f, pairs with l > original/low turn
+    ``factor`` times slower, and between the two f is blended with s =
+    (original/l - low) / (high - low): (1 - s) f / factor + s f.  float64;
+    callers round once to f32."""
+    import math
+
+    freqs = [float(base) ** (-2.0 * i / dims) for i in range(dims // 2)]
+    if not scaling:
+        return freqs
+    factor, low, high = float(scaling["factor"]), float(scaling["low"]), float(scaling["high"])
+    orig = float(scaling["original"])
+    out = []
+    for f in freqs:
+        wave = 2.0 * math.pi / f
+        if wave < orig / high:
+            out.append(f)
+        elif wave > orig / low:
+            out.append(f / factor)
+        else:
+            s = (orig / wave - low) / (high - low)
+            out.append((1.0 - s) * f / factor + s * f)
+    return out
+
+
+class DiffAttention(_Mixer):
+    """Differential grouped-query attention.
+
+    Every query head has two maps (two queries of ``dim`` each) and every
+    key/value head two keys and one value: each map is a causal softmax
+    attention of its own over the same values, a_1 and a_2, and the head's
+    output is (a_1 - lam a_2) / rms(a_1 - lam a_2) * (1 - diff) with lam =
+    exp(lq1 . lk1) - exp(lq2 . lk2) + diff, one number for the layer.
+    Queries and keys are RMS-normed per head and map (one weight for all of
+    them), then their first ``rot_dims`` dims are rotated (dim i with i +
+    rot_dims/2).  score = q . k * scale; with ``chunk`` > 0 position i sees j
+    <= i only inside its own chunk of that many positions.  Head h's output
+    is multiplied by sigmoid(W_g h)_h.
+
+    Projected rows: [q map 1 | q map 2 | k map 1 | k map 2 | v | gate] — the
+    maps are laid out as 2H query heads over 2G key heads, so that the usual
+    grouped-query rule (query head / (H / G)) finds the right key, and key
+    head g reads value head g mod G."""
+
+    def __init__(self, width: int, *, heads: int, kv_heads: int, dim: int, vdim: int,
+                 scale: float, diff: float, eps: float, chunk: int = 0,
+                 rot_base: float = 10000.0, rot_dims: int = 0,
+                 rot_scaling: Optional[dict] = None, head_gate: bool = True,
+                 own_in: bool = True, dtype: torch.dtype = torch.bfloat16):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        if rot_dims % 2 or rot_dims > dim:
+            raise ValueError("rot_dims must be even and at most dim")
+        self.heads, self.kv_heads, self.dim, self.vdim = heads, kv_heads, dim, vdim
+        self.scale, self.diff, self.eps, self.chunk = scale, diff, eps, chunk
+        self.rot_dims, self.head_gate = rot_dims, head_gate
+        self.in_rows = (2 * heads * dim + 2 * kv_heads * dim + kv_heads * vdim
+                        + (heads if head_gate else 0))
+        self.out_rows = heads * vdim
+        self._alloc(width, own_in, dtype)
+        self.q_norm = _f32_param(dim, fill=1.0)
+        self.k_norm = _f32_param(dim, fill=1.0)
+        self.lam = diff
+        freqs = stepped_rotary_frequencies(rot_base, max(rot_dims, 2), rot_scaling)
+        self.register_buffer(
+            "inv_freq", torch.tensor(freqs, dtype=torch.float64).to(torch.float32),
+            persistent=False)
+
+    def load_in(self, weight, bias, t) -> None:
+        nh, ng, d = self.heads, self.kv_heads, self.dim
+        # checkpoint rows are head by head [map 1, map 2]; here map by map
+        q = t["q"].view(nh, 2, d, -1).transpose(0, 1).reshape(2 * nh * d, -1)
+        k = t["k"].view(ng, 2, d, -1).transpose(0, 1).reshape(2 * ng * d, -1)
+        off = 0
+        for w in [q, k, t["v"]] + ([t["g"]] if self.head_gate else []):
+            weight[off:off + w.shape[0]].copy_(w.to(weight.dtype))
+            off += w.shape[0]
+        if off != self.in_rows:
+            raise ValueError("projection tensors do not add up to the mixer's rows")
+
+    def load_rest(self, t) -> None:
+        import math
+
+        self.q_norm.data.copy_(t["q.norm"].float())
+        self.k_norm.data.copy_(t["k.norm"].float())
+        dot = lambda a, b: float((t[a].double() * t[b].double()).sum())
+        self.lam = math.exp(dot("lq1", "lk1")) - math.exp(dot("lq2", "lk2")) + self.diff
+
+    def cache_shapes(self, block_size: int) -> list:
+        return [("paged", (block_size, 2 * self.kv_heads, self.dim), self.dtype),
+                ("paged", (block_size, self.kv_heads, self.vdim), self.dtype)]
+
+    def mix(self, proj, positions, cache, meta: AttnMetadata) -> torch.Tensor:
+        t = proj.shape[0]
+        nh, ng, d, dv = self.heads, self.kv_heads, self.dim, self.vdim
+        a = 2 * nh * d
+        b = a + 2 * ng * d
+        c = b + ng * dv
+        k_cache, v_cache = cache
+        q = ops.qk_norm_rope_cache_write(
+            proj[:, :a].view(t, 2 * nh, d), proj[:, a:b].view(t, 2 * ng, d),
+            proj[:, b:c].view(t, ng, dv), self.q_norm, self.k_norm, self.eps, positions,
+            self.inv_freq, self.rot_dims, k_cache, v_cache, meta.slot_mapping)
+        maps = torch.empty((t, 2 * nh, dv), dtype=torch.float32, device=proj.device)
+        npt = meta.num_prefill_tokens
+        if npt:
+            ops.chunk_attention_prefill(
+                q[:npt], k_cache, v_cache, meta.prefill_block_tables,
+                meta.prefill_query_start_loc, meta.prefill_seq_lens, self.scale,
+                meta.max_prefill_query_len, self.chunk, out=maps[:npt])
+        if meta.num_decode_seqs:
+            ops.chunk_attention_decode(
+                q[npt:], k_cache, v_cache, meta.decode_block_tables,
+                meta.decode_seq_lens, self.scale, self.chunk, out=maps[npt:])
+        return ops.diff_combine(maps.view(t, 2, nh, dv), self.lam, 1.0 - self.diff, self.eps,
+                                proj[:, c:] if self.head_gate else None, self.dtype)
+
+
+class HGRN2Mixer(_Mixer):
+    """Gated linear recurrence with a matrix state per head.  q = silu(W_q h),
+    v = W_v h, forget gate per head and channel g = l + (1 - l) sigmoid(W_f h +
+    b) with the lower bound l a weight; S_t = diag(g_t) S_(t-1) + (1 - g_t)
+    v_t^T, o_t = S_t^T q_t (no key: 1 - g plays its part); each head's o is
+    RMS-normed over vdim with one weight for all heads.  Projected rows:
+    [q | f | v]."""
+
+    def __init__(self, width: int, *, heads: int, dim: int, vdim: int, eps: float,
+                 own_in: bool = True, dtype: torch.dtype = torch.bfloat16):
+        super().__init__()
+        self.heads, self.dim, self.vdim, self.eps = heads, dim, vdim, eps
+        self.in_rows = 2 * heads * dim + heads * vdim
+        self.out_rows = heads * vdim
+        self._alloc(width, own_in, dtype)
+        self.f_bias = _f32_param(heads * dim)
+        self.lower = _f32_param(heads * dim)
+        self.norm = _f32_param(heads * vdim, fill=1.0)   # the head weight, repeated
+
+    def load_in(self, weight, bias, t) -> None:
+        off = 0
+        for name in ("q", "f", "v"):
+            n = t[name].shape[0]
+            weight[off:off + n].copy_(t[name].to(weight.dtype))
+            off += n
+        if off != self.in_rows:
+            raise ValueError("projection tensors do not add up to the mixer's rows")
+
+    def load_rest(self, t) -> None:
+        self.f_bias.data.copy_(t["f.b"].float())
+        self.lower.data.copy_(t["lower"].float())
+        self.norm.data.copy_(t["norm"].float().repeat(self.heads))
+
+    def cache_shapes(self, block_size: int) -> list:
+        return [("slot", (self.heads, self.vdim, self.dim), torch.float32)]
+
+    def mix(self, proj, positions, cache, meta: AttnMetadata) -> torch.Tensor:
+        t, nh, d, dv = proj.shape[0], self.heads, self.dim, self.vdim
+        a = nh * d
+        o = ops.hgrn2_scan(proj[:, :a].view(t, nh, d), proj[:, a:2 * a].view(t, nh, d),
+                           proj[:, 2 * a:].view(t, nh, dv), self.f_bias, self.lower,
+                           cache[0], meta.seq_start_loc, meta.seq_lens, meta.state_slots)
+        return ops.group_rms_norm(o, self.norm, nh, self.eps, self.dtype)
+
+
+class GatedRoutedExperts(nn.Module):
+    """Mixture of ``experts`` small feed-forwards down(silu(gate x) * (up x))
+    without biases.  Router: z = W_r h in f32, s = sigmoid(z); the ``top``
+    largest s are chosen and weigh their experts as they are (no
+    renormalising).  The weight multiplies the expert's *input*: y = sum
+    expert(s_e h).
+
+    Without biases gate (s h) = s (gate h), so the weight is applied to the
+    projected rows.  Two ways to run the experts, chosen by shape:
+
+    - stacked: one product with every expert's [gate ; up] rows stacked
+      [E * 2 ff, width], silu(s g) * (s u) with s = 0 for unchosen experts (they
+      vanish exactly), one product with the down-projections stacked along the
+      contraction axis.  Any size, f32 or bf16, shape-static.
+    - grouped: token-expert pairs grouped by expert, their rows multiplied by
+      s, one grouped gated product and one grouped down-projection over the
+      expert segments (bf16, sizes in multiples of 128), gather-sum."""
+
+    def __init__(self, width: int, *, experts: int, top: int, ff: int,
+                 dtype: torch.dtype, grouped: Optional[bool] = None):
+        super().__init__()
+        if get_tp_world_size() != 1:
+            raise ValueError("GatedRoutedExperts is not sharded; run it with one rank")
+        if not 1 <= top <= experts:
+            raise ValueError("top must lie between 1 and the number of experts")
+        self.width, self.experts, self.top, self.ff = width, experts, top, ff
+        self.dtype = dtype
+        fits = dtype == torch.bfloat16 and ff % 128 == 0 and width % 128 == 0
+        self.grouped = (fits and experts > 2 * top) if grouped is None else bool(grouped)
+        if self.grouped and not fits:
+            raise ValueError("grouped experts need bf16 and sizes in multiples of 128")
+        self.router = nn.Parameter(
+            torch.empty(experts, width, dtype=torch.float32).normal_(0.0, width ** -0.5),
+            requires_grad=False)
+        # per expert: ff gate rows, then ff up rows
+        self.gate_up = _randn_param((experts, 2 * ff, width), dtype, std=width ** -0.5)
+        if self.grouped:
+            self.down = _randn_param((experts, width, ff), dtype, std=ff ** -0.5)
+        else:
+            self.down = _randn_param((width, experts * ff), dtype, std=ff ** -0.5)
+
+    def load(self, router, gates: list, ups: list, downs: list) -> None:
+        self.router.data.copy_(router.float())
+        ff = self.ff
+        for e, (g, u, d) in enumerate(zip(gates, ups, downs)):
+            self.gate_up.data[e, :ff].copy_(g.to(self.dtype))
+            self.gate_up.data[e, ff:].copy_(u.to(self.dtype))
+            if self.grouped:
+                self.down.data[e].copy_(d.to(self.dtype))
+            else:
+                self.down.data[:, e * ff:(e + 1) * ff].copy_(d.to(self.dtype))
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        z = torch.nn.functional.linear(h.float(), self.router)
+        dense, ids, w = ops.moe_route_sigmoid(z, self.top)
+        ne = self.experts
+        if not self.grouped:
+            gu = ops.linear(h, self.gate_up.view(ne * 2 * self.ff, self.width))
+            return ops.linear(ops.silu_mul_scaled(gu, dense), self.down)
+        xs, pos, seg = ops.moe_sort(ids, ne, h, row_scale=w)
+        a = ops.moe_gemm(xs, self.gate_up, seg, gated=True)
+        ye = ops.moe_gemm(a, self.down, seg, gated=False)
+        return ops.moe_combine(ye, pos, ids, torch.ones_like(w), ne)

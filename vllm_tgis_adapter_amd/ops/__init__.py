@@ -561,24 +561,32 @@ def stream_add(x: torch.Tensor, a: torch.Tensor, b: torch.Tensor | None,
 
 
 def stream_add_rms_norm(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor,
-                        eps: float, mult: float, next_norm=None):
-    """x (f32, in place) += mult * y / rms(y) * weight.
+                        eps: float, mult: float, next_norm=None,
+                        layer_scale: torch.Tensor | None = None,
+                        cast_dtype: torch.dtype | None = None):
+    """x (f32, in place) += mult * y / rms(y) * weight (* layer_scale [W] f32).
 
     ``next_norm`` = (weight, eps, weight_offset, dtype) fuses the following
-    norm of the updated stream into the same pass and returns its output."""
+    norm of the updated stream into the same pass and returns its output;
+    ``cast_dtype`` instead returns the updated stream rounded to that dtype
+    (for a sublayer that reads the stream itself)."""
+    if next_norm is not None and cast_dtype is not None:
+        raise ValueError("either the next norm or a cast of the stream, not both")
     if x.numel() and _native_seq(x):
         if next_norm is None:
+            out = (torch.empty(x.shape, dtype=cast_dtype, device=x.device)
+                   if cast_dtype is not None else None)
             _S.stream_add_rms_norm(x, y, weight, float(eps), float(mult),
-                                   None, None, 0.0, 0.0)
-            return None
+                                   out, None, 0.0, 0.0, layer_scale)
+            return out
         nw, neps, noff, ndtype = next_norm
         out = torch.empty(x.shape, dtype=ndtype, device=x.device)
         _S.stream_add_rms_norm(x, y, weight, float(eps), float(mult), out, nw,
-                               float(neps), float(noff))
+                               float(neps), float(noff), layer_scale)
         return out
-    reference.stream_add_rms_norm(x, y, weight, eps, mult)
+    reference.stream_add_rms_norm(x, y, weight, eps, mult, layer_scale)
     if next_norm is None:
-        return None
+        return x.to(cast_dtype) if cast_dtype is not None else None
     nw, neps, noff, ndtype = next_norm
     return reference.rms_norm_stream(x, nw, neps, noff, ndtype)
 
@@ -1017,13 +1025,15 @@ def moe_combine(ye: torch.Tensor, pos: torch.Tensor, ids: torch.Tensor,
     return reference.moe_combine(ye, pos, ids, weights, num_real)
 
 
-def moe_sort(ids: torch.Tensor, num_real: int, h: torch.Tensor):
+def moe_sort(ids: torch.Tensor, num_real: int, h: torch.Tensor,
+             row_scale: torch.Tensor | None = None):
     """Group the token-expert pairs ids [T, top] by expert.  Returns (xs
     [T * top, W]: h's rows gathered so that expert e's pairs fill rows seg[e] ..
     seg[e+1], pos [T, top] int32: the row of each pair (0 for identity experts,
     ids >= num_real, which get no row), seg [num_real + 1] int32).  Rows past
     seg[-1] are left unwritten.  The order of the pairs inside a segment is
-    not specified."""
+    not specified.  ``row_scale`` [T, top] f32: pair (t, k)'s gathered row is
+    h[t] times row_scale[t, k], rounded once."""
     if h.numel() and _native_seq(h):
         t, top = ids.shape
         dev = h.device
@@ -1031,6 +1041,139 @@ def moe_sort(ids: torch.Tensor, num_real: int, h: torch.Tensor):
         pos = torch.empty((t, top), dtype=torch.int32, device=dev)
         seg = torch.empty((num_real + 1,), dtype=torch.int32, device=dev)
         scratch = torch.zeros((2 * num_real,), dtype=torch.int32, device=dev)
-        _S.moe_sort(xs, pos, seg, scratch, h, ids, int(num_real))
+        _S.moe_sort(xs, pos, seg, scratch, h, ids, int(num_real), row_scale)
         return xs, pos, seg
-    return reference.moe_sort(ids, num_real, h)
+    return reference.moe_sort(ids, num_real, h, row_scale)
+
+
+# ---------------------------------------------------------------------------
+# Token shift with per-sequence state, query/key norm + rotation + cache
+# write, chunk-masked attention with shared value heads and the differential
+# combination of two maps, the HGRN2 recurrence, sigmoid routing and gated
+# experts fed weighted inputs.  Same extension as the stream ops.
+# ---------------------------------------------------------------------------
+
+
+def token_shift_state(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor,
+                      seq_start_loc, seq_lens, state_slots,
+                      out_dtype: torch.dtype) -> torch.Tensor:
+    """x_t + (x_(t-1) - x_t) * weight over each sequence's new rows of the f32
+    stream, in the compute dtype; the row before a portion comes from
+    ``state[slot]`` (f32, zero before position 0), which then takes the
+    portion's last row."""
+    if x.numel() and _native_seq(x):
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        _S.token_shift_state(out, x, weight, state, seq_start_loc, seq_lens, state_slots)
+        return out
+    return reference.token_shift_state(x, weight, state, seq_start_loc.cpu(),
+                                       seq_lens.cpu(), state_slots.cpu(), out_dtype)
+
+
+def qk_norm_rope_cache_write(q, k, v, q_weight, k_weight, eps, positions, inv_freq,
+                             rot_dims: int, k_cache, v_cache, slot_mapping) -> torch.Tensor:
+    """Per-head RMS norm of q [T, H, dim] and k [T, G, dim] (views into a merged
+    projection are fine), rotation of the first ``rot_dims`` dims (dim i with
+    i + rot_dims/2) in f32, one rounding; keys and v [T, Gv, vdim] stored in the
+    paged cache.  Returns contiguous queries."""
+    if q.numel() and _native_seq(q):
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        _S.qk_norm_rope_cache_write(out, q, k, v, q_weight, k_weight, float(eps),
+                                    positions, inv_freq, int(rot_dims), k_cache,
+                                    v_cache, slot_mapping)
+        return out
+    return reference.qk_norm_rope_cache_write(q, k, v, q_weight, k_weight, eps, positions,
+                                              inv_freq, rot_dims, k_cache, v_cache,
+                                              slot_mapping)
+
+
+def chunk_attention_prefill(q, k_cache, v_cache, block_tables, query_start_loc,
+                            seq_lens, scale, max_query_len, chunk: int,
+                            out: torch.Tensor) -> torch.Tensor:
+    """Causal grouped-query softmax attention of query portions over the paged
+    cache where position i sees only the keys of its own chunk of ``chunk``
+    positions (counted from position 0; 0 = no chunks).  The value cache may
+    hold fewer heads than the key cache (key head g reads value head g mod
+    Gv).  out [T, H, vdim] f32."""
+    if q.numel() and _native_seq(q):
+        _S.chunk_attention(out, q, k_cache, v_cache, block_tables, query_start_loc,
+                           seq_lens, float(scale), int(max_query_len), int(chunk))
+        return out
+    out.copy_(reference.chunk_attention(q, k_cache, v_cache, block_tables.cpu(),
+                                        query_start_loc.cpu(), seq_lens.cpu(), scale, chunk))
+    return out
+
+
+def chunk_attention_decode(q, k_cache, v_cache, block_tables, seq_lens, scale,
+                           chunk: int, out: torch.Tensor) -> torch.Tensor:
+    """Same attention for one new query per sequence (length 0 = padding row)."""
+    if q.numel() and _native_seq(q):
+        _S.chunk_attention(out, q, k_cache, v_cache, block_tables, None, seq_lens,
+                           float(scale), 1, int(chunk))
+        return out
+    qsl = torch.arange(q.shape[0] + 1, dtype=torch.int32)
+    out.copy_(reference.chunk_attention(q, k_cache, v_cache, block_tables.cpu(), qsl,
+                                        seq_lens.cpu(), scale, chunk))
+    return out
+
+
+def diff_combine(a: torch.Tensor, lam: float, out_scale: float, eps: float,
+                 gate: torch.Tensor | None, out_dtype: torch.dtype) -> torch.Tensor:
+    """Differential attention's combination of two maps a [T, 2, H, vdim] f32:
+    (a0 - lam * a1) / rms over vdim * out_scale * sigmoid(gate[t, h]) ->
+    [T, H * vdim] in the compute dtype."""
+    if a.numel() and _native_seq(a):
+        t, _, h, dv = a.shape
+        out = torch.empty((t, h * dv), dtype=out_dtype, device=a.device)
+        _S.diff_combine(out, a, float(lam), float(out_scale), float(eps), gate)
+        return out
+    return reference.diff_combine(a, lam, out_scale, eps, gate, out_dtype)
+
+
+def hgrn2_scan(q, f, v, f_bias, lower, state, seq_start_loc, seq_lens,
+               state_slots) -> torch.Tensor:
+    """HGRN2 recurrence over each sequence's new rows, f32 state [slots, H,
+    vdim, dim] advanced in place; q, f [T, H, dim] and v [T, H, vdim] may be
+    views into a merged projection.  Returns o [T, H * vdim] f32."""
+    if q.numel() and _native_seq(q):
+        o = torch.empty((q.shape[0], q.shape[1] * v.shape[-1]), dtype=torch.float32,
+                        device=q.device)
+        _S.hgrn2_scan(o, q, f, v, f_bias, lower, state, seq_start_loc, seq_lens,
+                      state_slots)
+        return o
+    return reference.hgrn2_scan(q, f, v, f_bias, lower, state, seq_start_loc.cpu(),
+                                seq_lens.cpu(), state_slots.cpu())
+
+
+def group_rms_norm(y: torch.Tensor, weight: torch.Tensor, groups: int, eps: float,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    """RMS norm of f32 y [T, C] in ``groups`` equal parts, times weight [C]."""
+    if y.numel() and _native_seq(y):
+        out = torch.empty(y.shape, dtype=out_dtype, device=y.device)
+        _S.group_rms_norm(out, y, weight, int(groups), float(eps))
+        return out
+    return reference.group_rms_norm(y, weight, groups, eps, out_dtype)
+
+
+def moe_route_sigmoid(logits: torch.Tensor, top: int):
+    """Sigmoid router: the ``top`` largest sigmoid(logits) per row, weighted by
+    those scores as they are.  Returns (dense [T, E] f32, ids [T, top] int32,
+    weights [T, top] f32)."""
+    if logits.numel() and _native_seq(logits):
+        t, n = logits.shape
+        dev = logits.device
+        dense = torch.empty((t, n), dtype=torch.float32, device=dev)
+        ids = torch.empty((t, top), dtype=torch.int32, device=dev)
+        w = torch.empty((t, top), dtype=torch.float32, device=dev)
+        _S.moe_route_sigmoid(dense, ids, w, logits)
+        return dense, ids, w
+    return reference.moe_route_sigmoid(logits, top)
+
+
+def silu_mul_scaled(gu: torch.Tensor, col_scale: torch.Tensor) -> torch.Tensor:
+    """gu [T, E * 2 * ff] (per expert its gate rows, then its up rows) ->
+    [T, E * ff]: silu(w * gate) * (w * up), w = col_scale[t, expert] f32."""
+    if gu.numel() and _native_seq(gu):
+        out = torch.empty((gu.shape[0], gu.shape[1] // 2), dtype=gu.dtype, device=gu.device)
+        _S.silu_mul_scaled(out, gu, col_scale)
+        return out
+    return reference.silu_mul_scaled(gu, col_scale)

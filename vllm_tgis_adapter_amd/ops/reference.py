@@ -199,10 +199,14 @@ def stream_add(x: torch.Tensor, a: torch.Tensor, b: torch.Tensor | None,
 
 
 def stream_add_rms_norm(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor,
-                        eps: float, mult: float) -> None:
+                        eps: float, mult: float,
+                        layer_scale: torch.Tensor | None = None) -> None:
     yf = y.float()
     r = torch.rsqrt(yf.pow(2).mean(dim=-1, keepdim=True) + eps)
-    x.add_(yf * r * weight.float(), alpha=mult)
+    n = yf * r * weight.float()
+    if layer_scale is not None:
+        n = n * layer_scale.float()
+    x.add_(n, alpha=mult)
 
 
 def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
@@ -717,9 +721,11 @@ def moe_gemm(x: torch.Tensor, w: torch.Tensor, seg_off: torch.Tensor, gated: boo
     return out
 
 
-def moe_sort(ids: torch.Tensor, num_real: int, h: torch.Tensor):
-    """Token-expert pairs grouped by expert (stable): gathered rows, each
-    pair's row, segment offsets of the real experts."""
+def moe_sort(ids: torch.Tensor, num_real: int, h: torch.Tensor,
+             row_scale: torch.Tensor | None = None):
+    """Token-expert pairs grouped by expert (stable): gathered rows (times
+    row_scale[t, k] f32 when given), each pair's row, segment offsets of the
+    real experts."""
     t, top = ids.shape
     flat = ids.reshape(-1).long()
     order = torch.argsort(flat, stable=True)
@@ -729,5 +735,162 @@ def moe_sort(ids: torch.Tensor, num_real: int, h: torch.Tensor):
     seg = torch.zeros(num_real + 1, dtype=torch.int32, device=ids.device)
     seg[1:] = counts.cumsum(0).to(torch.int32)
     xs = h[torch.div(order, top, rounding_mode="floor")]
+    if row_scale is not None:
+        xs = (xs.float() * row_scale.reshape(-1)[order].float().unsqueeze(1)).to(h.dtype)
     pos = torch.where(flat < num_real, pos, torch.zeros_like(pos))
     return xs, pos.view(t, top).to(torch.int32), seg
+
+
+# ---------------------------------------------------------------------------
+# Token shift with per-sequence state, query/key norm followed by rotation,
+# chunk-masked differential attention, the HGRN2 recurrence, sigmoid routing
+# and gated experts whose input carries the routing weight.
+# ---------------------------------------------------------------------------
+
+
+def token_shift_state(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor,
+                      seq_start_loc, seq_lens, state_slots,
+                      out_dtype: torch.dtype) -> torch.Tensor:
+    """out_t = x_t + (x_(t-1) - x_t) * weight per sequence, x [T, W] f32; the
+    row before a portion's first row comes from ``state[slot]`` (f32 [slots,
+    W]), the row before position 0 is zero; ``state[slot]`` then becomes the
+    portion's last row."""
+    out = torch.zeros(x.shape, dtype=out_dtype, device=x.device)
+    wf = weight.float()
+    for a, b, start, slot in _seq_iter(seq_start_loc, seq_lens, state_slots):
+        if slot < 0:
+            continue
+        xs = x[a:b].float()
+        first = state[slot].float() if start > 0 else torch.zeros_like(xs[0])
+        prev = torch.cat([first.unsqueeze(0), xs[:-1]], dim=0)
+        out[a:b] = (xs + (prev - xs) * wf).to(out_dtype)
+        state[slot] = xs[-1]
+    return out
+
+
+def qk_norm_rope_cache_write(q, k, v, q_weight, k_weight, eps, positions, inv_freq,
+                             rot_dims: int, k_cache, v_cache, slot_mapping):
+    """Per-head RMS norm of q [T, H, dim] and k [T, G, dim] (plain weight),
+    then rotation of the first ``rot_dims`` dims (dim i with i + rot_dims/2,
+    f32 angles position * inv_freq[i]); rotated keys and v [T, Gv, vdim] go to
+    the paged cache.  Returns the queries, contiguous."""
+    def norm_rot(x, w):
+        xf = x.float()
+        xf = xf * torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + eps) * w.float()
+        if rot_dims:
+            xf = xf.contiguous()
+            rope_partial(xf, positions, inv_freq, 0, rot_dims)
+        return xf
+    qf, kf = norm_rot(q, q_weight), norm_rot(k, k_weight)
+    ok = slot_mapping >= 0
+    sm = slot_mapping[ok]
+    bs = k_cache.shape[1]
+    blk = torch.div(sm, bs, rounding_mode="floor")
+    k_cache[blk, sm % bs] = kf[ok].to(k_cache.dtype)
+    v_cache[blk, sm % bs] = v[ok].to(v_cache.dtype)
+    return qf.to(q.dtype).contiguous()
+
+
+def chunk_attention(q, k_cache, v_cache, block_tables, query_start_loc, seq_lens,
+                    scale: float, chunk: int) -> torch.Tensor:
+    """Causal grouped-query softmax attention of each sequence's tail rows over
+    the paged cache in which position i sees j <= i only when floor(i / chunk)
+    = floor(j / chunk) (chunk 0: every j <= i).  q [T, H, dim]; key head of
+    query head h is h // (H / G); the value cache may hold fewer heads Gv than
+    the key cache: key head g reads value head g % Gv.  Returns f32 [T, H,
+    vdim]."""
+    nh, ng, gv = q.shape[1], k_cache.shape[2], v_cache.shape[2]
+    group = nh // ng
+    out = torch.zeros((q.shape[0], nh, v_cache.shape[-1]), dtype=torch.float32,
+                      device=q.device)
+    qs = query_start_loc.tolist()
+    lens = seq_lens.tolist()
+    for i in range(len(lens)):
+        s, e = qs[i], qs[i + 1]
+        n, ctx = e - s, lens[i]
+        if n == 0 or ctx == 0:
+            continue
+        k, v = _gather_kv(k_cache, v_cache, block_tables[i], ctx)
+        kf = k.float().repeat_interleave(group, dim=1)
+        vh = torch.arange(nh, device=q.device) // group % gv
+        vf = v.float()[:, vh]
+        scores = torch.einsum("qhd,shd->hqs", q[s:e].float(), kf) * scale
+        kpos = torch.arange(ctx, device=q.device)
+        qpos = torch.arange(ctx - n, ctx, device=q.device)
+        mask = kpos[None, :] > qpos[:, None]
+        if chunk > 0:
+            mask = mask | (torch.div(qpos[:, None], chunk, rounding_mode="floor")
+                           != torch.div(kpos[None, :], chunk, rounding_mode="floor"))
+        scores.masked_fill_(mask.unsqueeze(0), float("-inf"))
+        out[s:e] = torch.einsum("hqs,shd->qhd", torch.softmax(scores, dim=-1), vf)
+    return out
+
+
+def diff_combine(a: torch.Tensor, lam: float, out_scale: float, eps: float,
+                 gate: torch.Tensor | None, out_dtype: torch.dtype) -> torch.Tensor:
+    """a [T, 2, H, vdim] f32, the two maps' outputs: o = a[:, 0] - lam * a[:, 1],
+    divided by its root mean square over vdim (eps inside the root), times
+    ``out_scale``, times sigmoid(gate[t, h]) when a gate [T, H] is given.
+    Returns [T, H * vdim]."""
+    o = a[:, 0].float() - lam * a[:, 1].float()
+    o = o * torch.rsqrt(o.pow(2).mean(dim=-1, keepdim=True) + eps) * out_scale
+    if gate is not None:
+        o = o * torch.sigmoid(gate.float()).unsqueeze(-1)
+    return o.to(out_dtype).reshape(o.shape[0], -1)
+
+
+def hgrn2_scan(q: torch.Tensor, f: torch.Tensor, v: torch.Tensor, f_bias: torch.Tensor,
+               lower: torch.Tensor, state: torch.Tensor, seq_start_loc, seq_lens,
+               state_slots) -> torch.Tensor:
+    """Gated linear recurrence whose forget gate also sets what is written.
+    q, f [T, H, dim] (projections, before their activations), v [T, H, vdim];
+    g = lower + (1 - lower) * sigmoid(f + f_bias) per channel; per head
+    S_t = diag(g_t) S_(t-1) + (1 - g_t) v_t^T, o_t = S_t^T silu(q_t).  State
+    [slots, H, vdim, dim] f32, advanced in place; a sequence that starts in
+    this step starts from zero.  Returns o [T, H * vdim] f32."""
+    t, nh, d = q.shape
+    dv = v.shape[-1]
+    qf = q.float()
+    qf = qf * torch.sigmoid(qf)
+    lo = lower.float().view(nh, d)
+    g = lo + (1.0 - lo) * torch.sigmoid(f.float() + f_bias.float().view(nh, d))
+    vf = v.float()
+    out = torch.zeros((t, nh, dv), dtype=torch.float32, device=q.device)
+    for a, b, start, slot in _seq_iter(seq_start_loc, seq_lens, state_slots):
+        if slot < 0:
+            continue
+        s = state[slot].clone() if start > 0 else torch.zeros_like(state[slot])
+        for i in range(a, b):
+            s = g[i].unsqueeze(1) * s + vf[i].unsqueeze(2) * (1.0 - g[i]).unsqueeze(1)
+            out[i] = torch.einsum("hvd,hd->hv", s, qf[i])
+        state[slot] = s
+    return out.view(t, nh * dv)
+
+
+def group_rms_norm(y: torch.Tensor, weight: torch.Tensor, groups: int, eps: float,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    """RMS norm of y [T, C] in ``groups`` equal parts, times weight [C]."""
+    t, c = y.shape
+    yg = y.float().view(t, groups, c // groups)
+    yg = yg * torch.rsqrt(yg.pow(2).mean(dim=-1, keepdim=True) + eps)
+    return (yg.reshape(t, c) * weight.float()).to(out_dtype)
+
+
+def moe_route_sigmoid(logits: torch.Tensor, top: int):
+    """s = sigmoid(logits) [T, E] f32; the ``top`` largest are chosen (ties:
+    the lower index); weights = their s as they are.  Returns (dense [T, E]
+    f32: weight or 0, ids [T, top] int32, weights [T, top] f32)."""
+    s = torch.sigmoid(logits.float())
+    order = torch.sort(s, dim=-1, descending=True, stable=True).indices[:, :top]
+    w = torch.gather(s, 1, order)
+    return torch.zeros_like(s).scatter_(1, order, w), order.to(torch.int32), w
+
+
+def silu_mul_scaled(gu: torch.Tensor, col_scale: torch.Tensor) -> torch.Tensor:
+    """gu [T, E, 2, ff] flattened (expert-major, gate rows then up rows);
+    out[t, e, j] = silu(w * gate) * (w * up) with w = col_scale[t, e]: the
+    gated activation of an expert whose input was multiplied by w."""
+    t, e = col_scale.shape
+    z = gu.float().view(t, e, 2, -1) * col_scale.float().view(t, e, 1, 1)
+    g, u = z[:, :, 0], z[:, :, 1]
+    return (g * torch.sigmoid(g) * u).to(gu.dtype).reshape(t, -1)
