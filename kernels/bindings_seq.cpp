@@ -41,6 +41,8 @@ void register_rec_ops(pybind11::module& m);
 // two-norm residual kernel, rotation + cache write, gates, squared relu,
 // expert router and combine (bindings_par.cpp)
 void register_par_ops(pybind11::module& m);
+// token shift, norm + rotation + cache write, chunk-masked attention, the
+// differential combination, HGRN2, weighted gated activation (bindings_mix.cpp)
 void register_mix_ops(pybind11::module& m);
 namespace {
 
@@ -295,4 +297,5 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("causal_conv_state", &causal_conv_state);
   register_rec_ops(m);
   register_par_ops(m);
+  register_mix_ops(m);
 }

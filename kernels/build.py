@@ -16,7 +16,9 @@ Several extensions, so that a model only builds the ones it uses
             convolution with per-sequence state, grouped-query attention of
             any shape, recurrences with per-sequence state, two-norm blocks,
             rotation + cache write, gates, expert routing, the grouped expert
-            product + bindings_seq.cpp, bindings_rec.cpp, bindings_par.cpp
+            product, token shift, chunk-masked differential attention pieces
+            + bindings_seq.cpp, bindings_rec.cpp, bindings_par.cpp,
+            bindings_mix.cpp
 ``_C_lat``  windowed latent attention with sinks + bindings_lat.cpp
 """
 
@@ -35,7 +37,8 @@ PKG = REPO / "vllm_tgis_adapter_amd"
 ARCH = os.environ.get("PYTORCH_ROCM_ARCH", "gfx950")
 
 _SEQ_SOURCES = ["stream_ops.hip", "canon_conv.hip", "layer_norm_stream.hip",
-                "paged_attention_any.hip", "recurrent_scan.hip", "gated_block.hip"]
+                "paged_attention_any.hip", "recurrent_scan.hip", "gated_block.hip",
+                "mix_ops.hip"]
 # kernels without torch types that more than one extension links
 _SHARED_SOURCES = ["moe_gemm.hip"]
 _LAT_SOURCES = ["latent_attention.hip", "latent_attention_mfma.hip"]
@@ -55,7 +58,7 @@ EXTENSIONS = {
     "_C_seq": dict(
         sources=lambda: [KERNELS / n for n in _SEQ_SOURCES + _SHARED_SOURCES]
         + [KERNELS / "bindings_seq.cpp", KERNELS / "bindings_rec.cpp",
-           KERNELS / "bindings_par.cpp"],
+           KERNELS / "bindings_par.cpp", KERNELS / "bindings_mix.cpp"],
     ),
     "_C_lat": dict(
         sources=lambda: [KERNELS / n for n in _LAT_SOURCES] + [KERNELS / "bindings_lat.cpp"],

@@ -7,8 +7,11 @@
 //
 // Query head h reads key/value head h / (H / G).  A query at position i sees
 // keys j with 0 <= i - j < window (window 0: every j <= i); with a sink the
-// softmax denominator also holds exp(sink), a key without a value.  One
-// workgroup per (query row, head).  Per tile of 256 keys:
+// softmax denominator also holds exp(sink), a key without a value; with a
+// chunk size c it sees only keys of its own chunk, floor(j / c) = floor(i / c),
+// chunks counted from position 0.  The value cache may hold fewer heads Gv
+// than the key cache: key head g reads value head g mod Gv.  The output type
+// may be f32 beside a 16-bit cache.  One workgroup per (query row, head).  Per tile of 256 keys:
 //   phase 1  thread j scores key j (q, already multiplied by the score scale,
 //            broadcast from LDS; the key row read with 16-byte loads), block
 //            max / sum give the online-softmax step
@@ -53,15 +56,15 @@ DEVINLINE float pa_reduce_sum(float x, float* scratch) {
   return s;
 }
 
-template <typename T>
+template <typename T, typename O>
 __global__ __launch_bounds__(PA_THREADS) void paged_attention_any_kernel(
-    T* __restrict__ out, long o_st, const T* __restrict__ q, long q_st,
+    O* __restrict__ out, long o_st, const T* __restrict__ q, long q_st,
     const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ qsl, const int* __restrict__ seq_lens, int nseq,
     float scale, int heads, int kv_heads, int dim, int vdim, int block_size,
     int vp /* pow2 >= min(vdim, 256) */, int vec_ok, int window, int has_sink,
-    float sink) {
+    float sink, int chunk, int v_heads) {
   extern __shared__ float smem[];
   float* q_s = smem;                               // [dim]
   float* p_s = q_s + ((dim + 1) & ~1);             // [256]
@@ -88,9 +91,10 @@ __global__ __launch_bounds__(PA_THREADS) void paged_attention_any_kernel(
     seq = row;
     ctx = seq_lens[row];
   }
-  T* orow = out + row * o_st + (long)h * vdim;
+  const int g_v = g_kv % v_heads;
+  O* orow = out + row * o_st + (long)h * vdim;
   if (ctx <= 0) {
-    for (int k = tid; k < vdim; k += PA_THREADS) orow[k] = ScalarOps<T>::from_f32(0.f);
+    for (int k = tid; k < vdim; k += PA_THREADS) orow[k] = ScalarOps<O>::from_f32(0.f);
     return;
   }
   const T* qr = q + row * q_st + (long)h * dim;
@@ -100,7 +104,7 @@ __global__ __launch_bounds__(PA_THREADS) void paged_attention_any_kernel(
   constexpr int V = Vec16<T>::kElems;
   const int* bt = block_tables + (long)seq * bt_stride;
   const long k_tok = (long)kv_heads * dim;     // elements per cached token
-  const long v_tok = (long)kv_heads * vdim;
+  const long v_tok = (long)v_heads * vdim;
 
   const int groups = PA_THREADS / vp;          // >= 1
   const int g = tid / vp;
@@ -110,7 +114,8 @@ __global__ __launch_bounds__(PA_THREADS) void paged_attention_any_kernel(
   for (int i = 0; i < PA_MAX_DPT; ++i) acc[i] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
 
-  const int first = (window > 0 && ctx > window) ? ctx - window : 0;
+  int first = (window > 0 && ctx > window) ? ctx - window : 0;
+  if (chunk > 0) first = max(first, ((ctx - 1) / chunk) * chunk);
   for (int base = first; base < ctx; base += PA_THREADS) {
     const int j = base + tid;
     float s = -INFINITY;
@@ -143,7 +148,7 @@ __global__ __launch_bounds__(PA_THREADS) void paged_attention_any_kernel(
     for (int i = 0; i < PA_MAX_DPT; ++i) acc[i] *= alpha;
     for (int jj = g; jj < nk; jj += groups) {
       const float pj = p_s[jj];
-      const T* vr = v_cache + tok_s[jj] * v_tok + (long)g_kv * vdim;
+      const T* vr = v_cache + tok_s[jj] * v_tok + (long)g_v * vdim;
 #pragma unroll
       for (int i = 0; i < PA_MAX_DPT; ++i) {
         const int k = k0 + i * vp;
@@ -166,18 +171,36 @@ __global__ __launch_bounds__(PA_THREADS) void paged_attention_any_kernel(
     if (g == 0 && k0 < vdim) {
       float a = 0.f;
       for (int gg = 0; gg < groups; ++gg) a += acc_s[gg * vp + k0];
-      orow[k0] = ScalarOps<T>::from_f32(a * inv);
+      orow[k0] = ScalarOps<O>::from_f32(a * inv);
     }
   } else {
 #pragma unroll
     for (int i = 0; i < PA_MAX_DPT; ++i) {
       const int k = k0 + i * vp;
-      if (k < vdim) orow[k] = ScalarOps<T>::from_f32(acc[i] * inv);
+      if (k < vdim) orow[k] = ScalarOps<O>::from_f32(acc[i] * inv);
     }
   }
 }
 
 }  // namespace
+
+template <typename T, typename O>
+static void launch_any(O* out, long o_st, const T* q, long q_st, const T* k_cache,
+                       const T* v_cache, const int* block_tables, int bt_stride,
+                       const int* qsl, const int* seq_lens, int nseq, float scale,
+                       int rows, int heads, int kv_heads, int dim, int vdim,
+                       int block_size, int vec_ok, int window, int has_sink,
+                       float sink, int chunk, int v_heads, hipStream_t stream) {
+  int vp = 1;
+  while (vp < vdim && vp < PA_THREADS) vp <<= 1;
+  const size_t smem = sizeof(float) * (((dim + 1) & ~1) + PA_THREADS + 16 + PA_THREADS) +
+                      sizeof(long) * PA_THREADS;
+  dim3 grid(rows, heads);
+  paged_attention_any_kernel<T, O><<<grid, PA_THREADS, smem, stream>>>(
+      out, o_st, q, q_st, k_cache, v_cache, block_tables, bt_stride, qsl,
+      seq_lens, nseq, scale, heads, kv_heads, dim, vdim, block_size, vp, vec_ok,
+      window, has_sink, sink, chunk, v_heads);
+}
 
 template <typename T>
 void launch_paged_attention_any(T* out, long o_st, const T* q, long q_st,
@@ -188,15 +211,23 @@ void launch_paged_attention_any(T* out, long o_st, const T* q, long q_st,
                                 int dim, int vdim, int block_size, int vec_ok,
                                 int window, int has_sink, float sink,
                                 hipStream_t stream) {
-  int vp = 1;
-  while (vp < vdim && vp < PA_THREADS) vp <<= 1;
-  const size_t smem = sizeof(float) * (((dim + 1) & ~1) + PA_THREADS + 16 + PA_THREADS) +
-                      sizeof(long) * PA_THREADS;
-  dim3 grid(rows, heads);
-  paged_attention_any_kernel<T><<<grid, PA_THREADS, smem, stream>>>(
-      out, o_st, q, q_st, k_cache, v_cache, block_tables, bt_stride, qsl,
-      seq_lens, nseq, scale, heads, kv_heads, dim, vdim, block_size, vp, vec_ok,
-      window, has_sink, sink);
+  launch_any<T, T>(out, o_st, q, q_st, k_cache, v_cache, block_tables, bt_stride, qsl,
+                   seq_lens, nseq, scale, rows, heads, kv_heads, dim, vdim,
+                   block_size, vec_ok, window, has_sink, sink, 0, kv_heads, stream);
+}
+
+// chunk-masked variant with f32 output and a value cache of v_heads heads
+template <typename T>
+void launch_chunk_attention(float* out, long o_st, const T* q, long q_st,
+                            const T* k_cache, const T* v_cache,
+                            const int* block_tables, int bt_stride, const int* qsl,
+                            const int* seq_lens, int nseq, float scale, int rows,
+                            int heads, int kv_heads, int v_heads, int dim, int vdim,
+                            int block_size, int vec_ok, int chunk,
+                            hipStream_t stream) {
+  launch_any<T, float>(out, o_st, q, q_st, k_cache, v_cache, block_tables, bt_stride,
+                       qsl, seq_lens, nseq, scale, rows, heads, kv_heads, dim, vdim,
+                       block_size, vec_ok, 0, 0, 0.f, chunk, v_heads, stream);
 }
 
 template void launch_paged_attention_any<float>(
@@ -207,3 +238,11 @@ template void launch_paged_attention_any<__hip_bfloat16>(
     __hip_bfloat16*, long, const __hip_bfloat16*, long, const __hip_bfloat16*,
     const __hip_bfloat16*, const int*, int, const int*, const int*, int, float,
     int, int, int, int, int, int, int, int, int, float, hipStream_t);
+template void launch_chunk_attention<float>(
+    float*, long, const float*, long, const float*, const float*, const int*, int,
+    const int*, const int*, int, float, int, int, int, int, int, int, int, int,
+    int, hipStream_t);
+template void launch_chunk_attention<__hip_bfloat16>(
+    float*, long, const __hip_bfloat16*, long, const __hip_bfloat16*,
+    const __hip_bfloat16*, const int*, int, const int*, const int*, int, float,
+    int, int, int, int, int, int, int, int, int, hipStream_t);

@@ -17,6 +17,11 @@
 //   KIND_MLSTM  log gates i, f (capped), running maximum m: alpha = exp(f + m
 //               - m'), beta = exp(i - m'), a normaliser n_t = alpha n + beta k,
 //               y = S q / (max(|n . q|, exp(-m')) + 1e-6)
+//   KIND_HGRN2  a forget gate per state channel that also sets what is
+//               written: S_t[j, i] = g_t[i] S_(t-1)[j, i] + (1 - g_t[i]) v_t[j],
+//               g = l + (1 - l) sigmoid(f + b) with a lower bound l per
+//               channel, y = S silu(q); a pointwise kernel ahead of the scan
+//               writes g and silu(q) in f32 once per (row, head, channel)
 // alpha, beta (and exp(-m')) are computed once per (row, head) by small gate
 // kernels ahead of the scan (for the mLSTM a sequential pass over the rows
 // carries the maximum), not by every thread of it.
@@ -34,10 +39,12 @@
 
 #include "common.h"
 
+#include <type_traits>
+
 namespace {
 
 constexpr int NPT = 16;   // state values per thread along N
-enum { KIND_SSD = 0, KIND_MLSTM = 1 };
+enum { KIND_SSD = 0, KIND_MLSTM = 1, KIND_HGRN2 = 2 };
 
 DEVINLINE float softplus_f(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
 DEVINLINE float logsigmoid_f(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
@@ -197,32 +204,36 @@ __global__ __launch_bounds__(256) void matrix_scan_kernel(ScanArgs a) {
 
   const float c2 = KIND == KIND_SSD ? a.p2[h] : 0.f;   // D
   const float4* gp = a.gates + h;
-  const T* qp = reinterpret_cast<const T*>(a.q) + (long)grp * a.nk;
-  const T* kp = reinterpret_cast<const T*>(a.k) + (long)grp * a.nk;
+  // HGRN2 reads its gate and activated query from the f32 rows of the pre-pass
+  using KQ = typename std::conditional<KIND == KIND_HGRN2, float, T>::type;
+  const KQ* qp = reinterpret_cast<const KQ*>(a.q) + (long)grp * a.nk;
+  const KQ* kp = reinterpret_cast<const KQ*>(a.k) + (long)grp * a.nk;
   const T* vp = reinterpret_cast<const T*>(a.v) + (long)h * a.vdim;
 
   for (int r = 0; r < n; ++r) {
     const long row = row0 + r;
     float kk[NPT], qq[NPT], vj[VPT];
-    load_slice<T>(kp + row * a.k_st, n0, a.nk, vec, kk);
-    load_slice<T>(qp + row * a.q_st, n0, a.nk, vec, qq);
+    load_slice<KQ>(kp + row * a.k_st, n0, a.nk, vec, kk);
+    load_slice<KQ>(qp + row * a.q_st, n0, a.nk, vec, qq);
 #pragma unroll
     for (int c = 0; c < VPT; ++c) vj[c] = ScalarOps<T>::to_f32(vp[row * a.v_st + jc[c]]);
-    const float4 gt = gp[row * a.heads];
+    const float4 gt = KIND == KIND_HGRN2 ? make_float4(0.f, 0.f, 0.f, 0.f)
+                                         : gp[row * a.heads];
     const float alpha = gt.x, beta = gt.y;
     float dot[VPT], ndot = 0.f;
 #pragma unroll
     for (int c = 0; c < VPT; ++c) dot[c] = 0.f;
 #pragma unroll
     for (int i = 0; i < NPT; ++i) {
-      const float bk = beta * kk[i];
+      const float al = KIND == KIND_HGRN2 ? kk[i] : alpha;
+      const float bk = KIND == KIND_HGRN2 ? 1.0f - kk[i] : beta * kk[i];
       if (KIND == KIND_MLSTM) {
         nst[i] = alpha * nst[i] + bk;
         ndot += nst[i] * qq[i];
       }
 #pragma unroll
       for (int c = 0; c < VPT; ++c) {
-        S[c][i] = alpha * S[c][i] + bk * vj[c];
+        S[c][i] = al * S[c][i] + bk * vj[c];
         dot[c] += S[c][i] * qq[i];
       }
     }
@@ -283,6 +294,23 @@ __global__ __launch_bounds__(256) void mlstm_norm_state_kernel(ScanArgs a) {
     }
     nrow[d] = nv;
   }
+}
+
+// HGRN2 pre-pass: gq [T, 2, H * dim] f32 = (l + (1 - l) sigmoid(f + b), silu(q))
+template <typename T>
+__global__ __launch_bounds__(256) void hgrn2_gates_kernel(
+    float* __restrict__ gq, const T* __restrict__ q, long q_st,
+    const T* __restrict__ f, long f_st, const float* __restrict__ f_bias,
+    const float* __restrict__ lower, long rows, int hd) {
+  const long idx = blockIdx.x * (long)blockDim.x + threadIdx.x;
+  if (idx >= rows * hd) return;
+  const long row = idx / hd;
+  const int c = (int)(idx - row * hd);
+  const float lo = lower[c];
+  const float fv = ScalarOps<T>::to_f32(f[row * f_st + c]) + f_bias[c];
+  const float qv = ScalarOps<T>::to_f32(q[row * q_st + c]);
+  gq[row * 2 * hd + c] = lo + (1.0f - lo) * sigmoid_f(fv);
+  gq[row * 2 * hd + hd + c] = qv * sigmoid_f(qv);
 }
 
 template <typename T, int KIND>
@@ -406,6 +434,30 @@ void launch_mlstm_scan(float* o, const T* q, long q_st, const T* k, long k_st,
 }
 
 template <typename T>
+void launch_hgrn2_scan(float* o, const T* q, long q_st, const T* f, long f_st,
+                       const T* v, long v_st, const float* f_bias,
+                       const float* lower, float* state, const int* loc,
+                       const int* seq_lens, const int* slots, int nseq, int heads,
+                       int dim, int vdim, int vec_ok, float* gq, int rows,
+                       hipStream_t stream) {
+  const int hd = heads * dim;
+  const long total = (long)rows * hd;
+  hgrn2_gates_kernel<T><<<(int)((total + 255) / 256), 256, 0, stream>>>(
+      gq, q, q_st, f, f_st, f_bias, lower, rows, hd);
+  ScanArgs a{};
+  a.rows = rows;
+  a.k = gq;      a.k_st = 2L * hd;
+  a.q = gq + hd; a.q_st = 2L * hd;
+  a.v = v;       a.v_st = v_st;
+  a.y = o; a.y_st = (long)heads * vdim;
+  a.s_state = state;
+  a.loc = loc; a.seq_lens = seq_lens; a.slots = slots;
+  a.heads = heads; a.vdim = vdim; a.nk = dim; a.per_group = 1;
+  a.vec_ok = vec_ok;
+  launch_matrix_scan<T, KIND_HGRN2>(a, nseq, stream);
+}
+
+template <typename T>
 void launch_rglru_scan(T* out, const T* u, const T* r_pre, const T* i_pre,
                        const float* r_bias, const float* i_bias, const float* lam,
                        float gate_c, const T* y_branch, float* state,
@@ -429,6 +481,11 @@ void launch_rglru_scan(T* out, const T* u, const T* r_pre, const T* i_pre,
       const T*, long, const float*, const float*, float, float, float*, float*, \
       float*, const int*, const int*, const int*, int, int, int, int, int,      \
       float*, int, hipStream_t);                                                \
+  template void launch_hgrn2_scan<T>(float*, const T*, long, const T*, long,    \
+                                     const T*, long, const float*, const float*,\
+                                     float*, const int*, const int*, const int*,\
+                                     int, int, int, int, int, float*, int,      \
+                                     hipStream_t);                              \
   template void launch_rglru_scan<T>(T*, const T*, const T*, const T*,          \
                                      const float*, const float*, const float*,  \
                                      float, const T*, float*, const int*,       \
