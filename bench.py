@@ -45,7 +45,8 @@ def parse_args():
     p.add_argument("--arch-sizes", type=str, default="s,m",
                    help="arch mode: comma list of sizes (s, m)")
     p.add_argument("--arch-models", type=str, default="dolodra,llama",
-                   help="arch mode: which models to run (dolodra, kezunex, relerax, llama)")
+                   help="arch mode: which models to run (dolodra, kezunex, relerax, gumozen, "
+                        "llama)")
     p.add_argument("--model", type=str, default="llama-3-8b")
     p.add_argument("--batch", type=int, default=512)
     p.add_argument("--prompt-len", type=int, default=512)
@@ -602,6 +603,50 @@ def _relerax_model_config(name: str, sz: dict, dtype: str):
     return mc
 
 
+# Gumozen at the same widths: eight post-norm layers [hgrn2, latent, attention,
+# latent borrowing the rows of the one before] x 2, every one followed by routed
+# gated experts whose chosen ones add up to about the llama's feed-forward.
+# HGRN2 heads of 128 x 128 (width / 128 heads); differential attention with
+# half the llama's head counts (each head has two maps of 128) and chunks of
+# 2048; latent attention with the latent of the Dolodra config and queries
+# through a latent three times as wide.
+GUMOZEN_SIZES = {
+    "s": dict(experts=16, top=4, expert_ff=1408, chunk=2048),
+    "m": dict(experts=16, top=4, expert_ff=3584, chunk=2048),
+    "t": dict(experts=4, top=2, expert_ff=48, chunk=24),
+}
+
+
+def _gumozen_model_config(name: str, sz: dict, dtype: str):
+    from vllm_tgis_adapter_amd.engine.config import _DTYPES
+    from vllm_tgis_adapter_amd.models.gumozen import model_config_from_json
+
+    gz = GUMOZEN_SIZES[name]
+    hd = sz["width"] // sz["heads"]
+    rec = {"heads": sz["heads"], "dim": hd, "vdim": hd}
+    att = {"heads": max(sz["heads"] // 2, 1), "kv_heads": max(sz["llama_kv_heads"] // 2, 1),
+           "dim": hd, "vdim": hd, "scale": hd ** -0.5, "diff": 0.3,
+           "mask": {"size": gz["chunk"]},
+           "rot": {"base": 10000.0, "dims": hd,
+                   "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 2048}}}
+    lat = {"heads": sz["heads"], "dim": sz["dim"], "vdim": sz["vdim"], "kv_rank": sz["rank"],
+           "q_rank": 3 * sz["rank"], "scale": sz["dim"] ** -0.5}
+    moe = {"kind": "moe", "expert": {"ff": gz["expert_ff"]},
+           "router": {"experts": gz["experts"], "top": gz["top"]}}
+    layers = []
+    for i in range(sz["layers"]):
+        kind = ("hgrn2", "latent_attention", "attention", "latent_attention")[i % 4]
+        mixer = dict({"hgrn2": rec, "attention": att, "latent_attention": lat}[kind])
+        if i % 4 == 3:
+            mixer["kv_from"] = i - 2
+        layers.append({"type": kind, "mixer": mixer, "mlp": moe})
+    hf = {"architecture": "Gumozen", "vocab": sz["vocab"], "width": sz["width"],
+          "layers": layers, "norm": {"eps": 1e-6}}
+    mc = model_config_from_json("gumozen-synthetic", hf)
+    mc.dtype = _DTYPES[dtype]
+    return mc
+
+
 def _arch_measure(mc, args, device: str, batch: int, prompt_len: int, steps: int,
                   warmup: int) -> dict:
     from vllm_tgis_adapter_amd.engine import EngineConfig, LLMEngine, SamplingParams
@@ -667,7 +712,8 @@ def run_arch(args, device: str) -> None:
         plen = args.prompt_len if device == "cuda" else 32
         steps = args.steps if device == "cuda" else 4
         warm = args.warmup if device == "cuda" else 1
-        models = [("dolodra", dolo), ("kezunex", None), ("relerax", None), ("llama", llama)]
+        models = [("dolodra", dolo), ("kezunex", None), ("relerax", None), ("gumozen", None),
+                  ("llama", llama)]
         for label, mc in models:
             if label not in args.arch_models.split(","):
                 continue
@@ -675,6 +721,8 @@ def run_arch(args, device: str) -> None:
                 mc = _kezunex_model_config(name, sz, args.dtype)
             if label == "relerax":
                 mc = _relerax_model_config(name, sz, args.dtype)
+            if label == "gumozen":
+                mc = _gumozen_model_config(name, sz, args.dtype)
             r = _arch_measure(mc, args, device, batch, plen, steps, warm)
             r.update(size=name, model=label, batch=batch, prompt_len=plen)
             out.append(r)

@@ -45,7 +45,10 @@ DEVINLINE bf16x8_t load_kv8<unsigned char>(const unsigned char* p) {
 // `window` keys only (window 0: all), and the probabilities enter the value
 // product as the sum of two bf16 terms (rounded value + rounded remainder);
 // the sink joins the denominator in the merge kernel.
-template <int HEAD_DIM, typename CT, bool WS>
+// CH (chunk variant, on top of WS): the query sees the keys of its own chunk
+// of `chunk` positions only; the value cache holds v_heads <= kvh heads and
+// key head g reads value head g mod v_heads.
+template <int HEAD_DIM, typename CT, bool WS, bool CH = false>
 __global__ __launch_bounds__(256, 2) void paged_decode_mfma_kernel(
     float* __restrict__ part_acc,   // [nseq, nheads, P, HEAD_DIM] f32
     float* __restrict__ part_ml,    // [nseq, nheads, P, 2] f32 (m, l)
@@ -60,7 +63,10 @@ __global__ __launch_bounds__(256, 2) void paged_decode_mfma_kernel(
     const int group,       // nheads / kvh, <= 8
     const int block_size,
     const int max_blocks,
-    const int window) {
+    const int window,
+    const int chunk = 0,
+    const int v_heads = 0) {
+  static_assert(!CH || WS, "the chunk variant builds on the window variant");
   constexpr int KCH = HEAD_DIM / 16;  // k-chunks for the QK^T mfma
   constexpr int DT = HEAD_DIM / 32;   // 32-col output tiles
 
@@ -78,7 +84,8 @@ __global__ __launch_bounds__(256, 2) void paged_decode_mfma_kernel(
 
   // this partition's tile range; waves stride by NWAVES inside it
   const int tiles_total = (seq_len + KVT - 1) / KVT;
-  const int first_pos = (WS && window > 0) ? max(0, seq_len - window) : 0;
+  const int first_pos = (CH && chunk > 0) ? max(0, seq_len - 1) / chunk * chunk
+                        : (WS && window > 0) ? max(0, seq_len - window) : 0;
   const int tile_first = first_pos / KVT;
   const int tpp = (tiles_total - tile_first + npart - 1) / npart;
   const int tile_lo = tile_first + part * tpp;
@@ -87,6 +94,8 @@ __global__ __launch_bounds__(256, 2) void paged_decode_mfma_kernel(
   const int head0 = kv_head * group;
   const int* btable = block_tables + (long)seq * max_blocks;
   const long kv_row_stride = (long)kvh * HEAD_DIM;
+  const long v_row_stride = CH ? (long)v_heads * HEAD_DIM : kv_row_stride;
+  const int v_head = CH ? kv_head % v_heads : kv_head;
 
   // per-wave V staging tile (linear; the B gather reads rows across lanes)
   __shared__ __hip_bfloat16 v_lds_all[NWAVES * KVT * HEAD_DIM];
@@ -151,8 +160,8 @@ __global__ __launch_bounds__(256, 2) void paged_decode_mfma_kernel(
         if (pos < seq_len) {
           const int block = btable[pos / block_size];
           const long row = ((long)block * block_size + pos % block_size) *
-                               kv_row_stride +
-                           (long)kv_head * HEAD_DIM + d8;
+                               v_row_stride +
+                           (long)v_head * HEAD_DIM + d8;
           vv[pass] = load_kv8<CT>(v_cache + row);
         }
       }
@@ -276,9 +285,9 @@ __global__ __launch_bounds__(256, 2) void paged_decode_mfma_kernel(
 }
 
 // Reduce the P partials of each (seq, head) row: out = sum_p f_p acc_p / sum_p f_p l_p
-template <int HEAD_DIM>
+template <int HEAD_DIM, typename OT = __hip_bfloat16>
 __global__ void decode_merge_kernel(
-    __hip_bfloat16* __restrict__ out,      // [nseq, nheads, HD]
+    OT* __restrict__ out,                  // [nseq, nheads, HD]
     const float* __restrict__ part_acc,    // [nseq, nheads, P, HD]
     const float* __restrict__ part_ml,     // [nseq, nheads, P, 2]
     const int nheads,
@@ -305,7 +314,10 @@ __global__ void decode_merge_kernel(
     A += f * acc[(long)p * HEAD_DIM];
   }
   const float inv = L > 0.f ? 1.f / L : 0.f;
-  out[row * HEAD_DIM + d] = __float2bfloat16(A * inv);
+  if constexpr (sizeof(OT) == 4)
+    out[row * HEAD_DIM + d] = A * inv;
+  else
+    out[row * HEAD_DIM + d] = __float2bfloat16(A * inv);
 }
 
 int decode_mfma_num_partitions(int nseq, int kvh, int max_context) {
@@ -411,4 +423,39 @@ void launch_paged_decode_mfma_ws(__hip_bfloat16* out, float* part_acc,
                                    scale, nseq, nheads, kvh, head_dim,
                                    block_size, max_blocks, npart, stream, window,
                                    has_sink, sink, true);
+}
+
+// chunk variant with shared value heads and f32 output (bf16 cache)
+void launch_paged_decode_mfma_chunk(float* out, float* part_acc, float* part_ml,
+                                    const __hip_bfloat16* q,
+                                    const __hip_bfloat16* kc,
+                                    const __hip_bfloat16* vc, const int* bt,
+                                    const int* sl, float scale, int nseq,
+                                    int nheads, int kvh, int v_heads, int head_dim,
+                                    int block_size, int max_blocks, int npart,
+                                    int chunk, hipStream_t stream) {
+  const int group = nheads / kvh;
+  dim3 grid(nseq, kvh, npart);
+  dim3 mgrid(nseq, nheads);
+  const int P = npart * NWAVES;
+  switch (head_dim) {
+    case 64:
+      hipLaunchKernelGGL(
+          (paged_decode_mfma_kernel<64, __hip_bfloat16, true, true>), grid, dim3(256),
+          0, stream, part_acc, part_ml, q, kc, vc, bt, sl, scale, nheads, kvh, group,
+          block_size, max_blocks, 0, chunk, v_heads);
+      hipLaunchKernelGGL((decode_merge_kernel<64, float>), mgrid, dim3(64), 0, stream,
+                         out, part_acc, part_ml, nheads, P, 0, 0.f);
+      break;
+    case 128:
+      hipLaunchKernelGGL(
+          (paged_decode_mfma_kernel<128, __hip_bfloat16, true, true>), grid,
+          dim3(256), 0, stream, part_acc, part_ml, q, kc, vc, bt, sl, scale, nheads,
+          kvh, group, block_size, max_blocks, 0, chunk, v_heads);
+      hipLaunchKernelGGL((decode_merge_kernel<128, float>), mgrid, dim3(128), 0,
+                         stream, out, part_acc, part_ml, nheads, P, 0, 0.f);
+      break;
+    default:
+      abort();
+  }
 }

@@ -63,9 +63,14 @@ __device__ inline float cross_half_sum(float v) {
 // also holds exp(sink); and the probabilities enter the value product as the
 // sum of two bf16 terms (rounded value + rounded remainder), so that they
 // carry 16 mantissa bits instead of 8.
-template <int HEAD_DIM, typename CT, int NW, bool WS>
+// CH (chunk variant, on top of WS with window 0): a query at position i sees
+// keys j <= i of its own chunk only, floor(j / chunk) = floor(i / chunk); the
+// value cache holds v_heads <= kvh heads and key head g reads value head
+// g mod v_heads; the output is f32.
+template <int HEAD_DIM, typename CT, int NW, bool WS, bool CH = false,
+          typename OT = __hip_bfloat16>
 __global__ __launch_bounds__(NW * 64, 512 / (NW * 64)) void paged_prefill_mfma_v2_kernel(
-    __hip_bfloat16* __restrict__ out,            // [total_q, nheads, HD]
+    OT* __restrict__ out,                        // [total_q, nheads, HD]
     const __hip_bfloat16* __restrict__ q,        // [total_q, nheads, HD]
     const CT* __restrict__ k_cache,  // [nb, bs, kvh, HD] bf16 | e4m3
     const CT* __restrict__ v_cache,
@@ -79,8 +84,11 @@ __global__ __launch_bounds__(NW * 64, 512 / (NW * 64)) void paged_prefill_mfma_v
     const int max_blocks,
     const int window,
     const int has_sink,
-    const float sink) {
+    const float sink,
+    const int chunk = 0,
+    const int v_heads = 0) {
   static_assert(HEAD_DIM == 128, "v2 is specialised for HD=128");
+  static_assert(!CH || WS, "the chunk variant builds on the window variant");
   constexpr int KCH = HEAD_DIM / 16;  // QK^T k-chunks (8)
   constexpr int DT = HEAD_DIM / 32;   // 32-col output tiles (4)
   constexpr int QT = NW * 32;         // q rows per workgroup
@@ -107,6 +115,8 @@ __global__ __launch_bounds__(NW * 64, 512 / (NW * 64)) void paged_prefill_mfma_v
 
   const int* btable = block_tables + (long)seq * max_blocks;
   const long kv_row_stride = (long)kvh * HEAD_DIM;
+  const long v_row_stride = CH ? (long)v_heads * HEAD_DIM : kv_row_stride;
+  const int v_head = CH ? kv_head % v_heads : kv_head;
 
   // K: [64][256B] XOR-swizzled; V: 16 x 1152B subtiles
   __shared__ __hip_bfloat16 k_lds2[2][KVT2 * HEAD_DIM];
@@ -116,6 +126,8 @@ __global__ __launch_bounds__(NW * 64, 512 / (NW * 64)) void paged_prefill_mfma_v
   const int q_row_local = tile_base + wave * 32 + col;
   const bool q_valid = q_row_local < q_len;
   const int q_pos = seq_len - q_len + q_row_local;
+  // first key position of the row's chunk
+  const int q_lo = (CH && chunk > 0 && q_valid) ? q_pos / chunk * chunk : 0;
   bf16x8_t qb[KCH];
   if (q_valid) {
     const __hip_bfloat16* q_row =
@@ -149,6 +161,10 @@ __global__ __launch_bounds__(NW * 64, 512 / (NW * 64)) void paged_prefill_mfma_v
     kv_first = max(0, seq_len - q_len + tile_base - window + 1) / KVT2 * KVT2;
     wave_win_lo = max(0, wave_q_pos_min - window + 1);
   }
+  if (CH && chunk > 0) {
+    kv_first = ((seq_len - q_len + tile_base) / chunk * chunk) / KVT2 * KVT2;
+    wave_win_lo = wave_q_pos_min / chunk * chunk;
+  }
 
   // ---- staging map: thread t covers slot (t % ROWS_PER_PASS, t / RPP * 8)
   // with ROWS_PER_PASS = NTHREADS/16 rows per pass (16 8-elem slots per row)
@@ -165,11 +181,11 @@ __global__ __launch_bounds__(NW * 64, 512 / (NW * 64)) void paged_prefill_mfma_v
       st_v[pass] = bf16x8_t{};
       if (pos < kv_limit) {
         const int block = btable[pos / block_size];
-        const long row = ((long)block * block_size + pos % block_size) *
-                             kv_row_stride +
-                         (long)kv_head * HEAD_DIM + st_d8;
-        st_k[pass] = load_kv8_v2<CT>(k_cache + row);
-        st_v[pass] = load_kv8_v2<CT>(v_cache + row);
+        const long tok = (long)block * block_size + pos % block_size;
+        st_k[pass] = load_kv8_v2<CT>(k_cache + tok * kv_row_stride +
+                                     (long)kv_head * HEAD_DIM + st_d8);
+        st_v[pass] = load_kv8_v2<CT>(v_cache + tok * v_row_stride +
+                                     (long)v_head * HEAD_DIM + st_d8);
       }
     }
   };
@@ -234,7 +250,9 @@ __global__ __launch_bounds__(NW * 64, 512 / (NW * 64)) void paged_prefill_mfma_v
                              (kv_base + KVT2 <= seq_len) &&
                              (tile_base + wave * 32 + 31 < q_len) &&
                              (!WS || window == 0 ||
-                              kv_base > wave_q_pos_min + 31 - window);
+                              kv_base > wave_q_pos_min + 31 - window) &&
+                             (!CH || chunk == 0 ||
+                              kv_base >= (wave_q_pos_min + 31) / chunk * chunk);
       float local_max = -FLT_MAX;
       if (full_tile) {
 #pragma unroll
@@ -251,7 +269,8 @@ __global__ __launch_bounds__(NW * 64, 512 / (NW * 64)) void paged_prefill_mfma_v
                 kv_base + kb * 32 + (r & 3) + 8 * (r >> 2) + 4 * half;
             float v = acc_s[kb][r];
             if (!q_valid || kv_pos > q_pos || kv_pos >= seq_len ||
-                (WS && window > 0 && kv_pos + window <= q_pos))
+                (WS && window > 0 && kv_pos + window <= q_pos) ||
+                (CH && kv_pos < q_lo))
               v = -FLT_MAX;
             acc_s[kb][r] = v;
             local_max = fmaxf(local_max, v);
@@ -390,11 +409,14 @@ __global__ __launch_bounds__(NW * 64, 512 / (NW * 64)) void paged_prefill_mfma_v
     const float l_inv = __shfl(l_inv_own, qrow, 64);
     const int q_local = tile_base + wave * 32 + qrow;
     if (q_local >= q_len) continue;
-    __hip_bfloat16* out_row =
-        out + ((long)(q_start + q_local) * nheads + head) * HEAD_DIM;
+    OT* out_row = out + ((long)(q_start + q_local) * nheads + head) * HEAD_DIM;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-      out_row[dt * 32 + col] = __float2bfloat16(acc_o[dt][r] * l_inv);
+    for (int dt = 0; dt < DT; ++dt) {
+      if constexpr (CH)
+        out_row[dt * 32 + col] = acc_o[dt][r] * l_inv;
+      else
+        out_row[dt * 32 + col] = __float2bfloat16(acc_o[dt][r] * l_inv);
+    }
   }
 }
 
@@ -469,4 +491,17 @@ void launch_paged_prefill_mfma_v2_ws(
                                        nseq, nheads, kvh, head_dim,
                                        block_size, max_blocks, max_query_len,
                                        stream, window, has_sink, sink, true);
+}
+
+// chunk variant with shared value heads and f32 output (bf16 cache, HD = 128)
+void launch_paged_prefill_mfma_v2_chunk(
+    float* out, const __hip_bfloat16* q, const __hip_bfloat16* kc,
+    const __hip_bfloat16* vc, const int* bt, const int* qsl, const int* sl,
+    float scale, int nseq, int nheads, int kvh, int v_heads, int block_size,
+    int max_blocks, int max_query_len, int chunk, hipStream_t stream) {
+  const int qtiles = (max_query_len + 255) / 256;
+  hipLaunchKernelGGL(
+      (paged_prefill_mfma_v2_kernel<128, __hip_bfloat16, 8, true, true, float>),
+      dim3(nseq, nheads, qtiles), dim3(512), 0, stream, out, q, kc, vc, bt, qsl,
+      sl, scale, nheads, kvh, block_size, max_blocks, 0, 0, 0.f, chunk, v_heads);
 }

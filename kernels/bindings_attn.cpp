@@ -48,6 +48,15 @@ void launch_paged_prefill_mfma_v2_ws(__hip_bfloat16*, const __hip_bfloat16*,
                                      const int*, const int*, const int*, float,
                                      int, int, int, int, int, int, int, int, int,
                                      float, hipStream_t);
+void launch_paged_prefill_mfma_v2_chunk(float*, const __hip_bfloat16*,
+                                        const __hip_bfloat16*, const __hip_bfloat16*,
+                                        const int*, const int*, const int*, float,
+                                        int, int, int, int, int, int, int, int,
+                                        hipStream_t);
+void launch_paged_decode_mfma_chunk(float*, float*, float*, const __hip_bfloat16*,
+                                    const __hip_bfloat16*, const __hip_bfloat16*,
+                                    const int*, const int*, float, int, int, int,
+                                    int, int, int, int, int, int, hipStream_t);
 void launch_paged_decode_mfma_ws(__hip_bfloat16*, float*, float*,
                                  const __hip_bfloat16*, const __hip_bfloat16*,
                                  const __hip_bfloat16*, const int*, const int*,
@@ -307,9 +316,93 @@ void windowed_attention_decode(torch::Tensor out, torch::Tensor q,
       has_sink ? 1 : 0, (float)sink, current_stream());
 }
 
+// Chunk variants of the bf16 MFMA kernels: position i sees keys j <= i with
+// floor(j / chunk) = floor(i / chunk) (0: all j <= i); the value cache may hold
+// fewer heads than the key cache (key head g reads value head g mod Gv); the
+// output is f32.  Sizes as for the window variants.
+void check_chunked(const torch::Tensor& out, const torch::Tensor& q,
+                   const torch::Tensor& k_cache, const torch::Tensor& v_cache,
+                   const torch::Tensor& block_tables, const torch::Tensor& seq_lens,
+                   int64_t chunk) {
+  TORCH_CHECK(q.is_cuda() && q.dim() == 3 && q.is_contiguous() && out.is_cuda() &&
+              out.is_contiguous() && out.sizes() == q.sizes(),
+              "q / out must be contiguous [rows, heads, dim]");
+  TORCH_CHECK(q.scalar_type() == at::ScalarType::BFloat16 &&
+              out.scalar_type() == at::ScalarType::Float &&
+              k_cache.scalar_type() == at::ScalarType::BFloat16 &&
+              v_cache.scalar_type() == at::ScalarType::BFloat16, "bf16 in, f32 out");
+  TORCH_CHECK(k_cache.is_cuda() && v_cache.is_cuda() && k_cache.is_contiguous() &&
+              v_cache.is_contiguous() && k_cache.dim() == 4 && v_cache.dim() == 4 &&
+              k_cache.size(0) == v_cache.size(0) && k_cache.size(1) == v_cache.size(1) &&
+              k_cache.size(3) == q.size(2) && v_cache.size(3) == q.size(2),
+              "cache shape");
+  const int nheads = q.size(1), kvh = k_cache.size(2), vh = v_cache.size(2);
+  TORCH_CHECK(kvh >= 1 && nheads % kvh == 0 && nheads / kvh <= 8, "heads per key head");
+  TORCH_CHECK(vh >= 1 && kvh % vh == 0, "key heads per value head");
+  TORCH_CHECK(block_tables.is_cuda() && block_tables.scalar_type() == at::ScalarType::Int &&
+              block_tables.dim() == 2 && block_tables.is_contiguous() &&
+              block_tables.size(0) >= seq_lens.numel());
+  TORCH_CHECK(seq_lens.is_cuda() && seq_lens.scalar_type() == at::ScalarType::Int &&
+              seq_lens.is_contiguous());
+  TORCH_CHECK(chunk >= 0, "chunk");
+}
+
+void chunk_attention_prefill(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
+                             torch::Tensor v_cache, torch::Tensor block_tables,
+                             torch::Tensor query_start_loc, torch::Tensor seq_lens,
+                             double scale, int64_t max_query_len, int64_t chunk) {
+  check_chunked(out, q, k_cache, v_cache, block_tables, seq_lens, chunk);
+  TORCH_CHECK(q.size(2) == 128, "prompt portions need key size 128");
+  const int nseq = seq_lens.numel();
+  TORCH_CHECK(query_start_loc.is_cuda() && query_start_loc.is_contiguous() &&
+              query_start_loc.scalar_type() == at::ScalarType::Int &&
+              query_start_loc.numel() == nseq + 1 && max_query_len >= 1);
+  if (q.size(0) == 0 || nseq == 0) return;
+  launch_paged_prefill_mfma_v2_chunk(
+      out.data_ptr<float>(), reinterpret_cast<const __hip_bfloat16*>(q.data_ptr()),
+      reinterpret_cast<const __hip_bfloat16*>(k_cache.data_ptr()),
+      reinterpret_cast<const __hip_bfloat16*>(v_cache.data_ptr()),
+      block_tables.data_ptr<int>(), query_start_loc.data_ptr<int>(),
+      seq_lens.data_ptr<int>(), (float)scale, nseq, (int)q.size(1),
+      (int)k_cache.size(2), (int)v_cache.size(2), (int)k_cache.size(1),
+      (int)block_tables.size(1), (int)max_query_len, (int)chunk, current_stream());
+}
+
+void chunk_attention_decode(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache,
+                            torch::Tensor v_cache, torch::Tensor block_tables,
+                            torch::Tensor seq_lens, double scale, int64_t chunk) {
+  check_chunked(out, q, k_cache, v_cache, block_tables, seq_lens, chunk);
+  const int nseq = q.size(0), nheads = q.size(1), head_dim = q.size(2);
+  TORCH_CHECK(head_dim == 64 || head_dim == 128, "key size 64 or 128");
+  TORCH_CHECK(seq_lens.numel() == nseq, "one query row per sequence expected");
+  if (nseq == 0) return;
+  const int kvh = k_cache.size(2), block_size = k_cache.size(1);
+  const int max_blocks = block_tables.size(1);
+  // shape-pure split count; a chunk bounds the keys a query reads
+  int span = max_blocks * block_size;
+  if (chunk > 0 && chunk + 32 < span) span = (int)chunk + 32;
+  const int npart = decode_mfma_num_partitions(nseq, kvh, span);
+  const int P = npart * 4;
+  auto opts = q.options().dtype(at::ScalarType::Float);
+  auto part_acc = at::empty({nseq, nheads, P, head_dim}, opts);
+  auto part_ml = at::empty({nseq, nheads, P, 2}, opts);
+  launch_paged_decode_mfma_chunk(
+      out.data_ptr<float>(), part_acc.data_ptr<float>(), part_ml.data_ptr<float>(),
+      reinterpret_cast<const __hip_bfloat16*>(q.data_ptr()),
+      reinterpret_cast<const __hip_bfloat16*>(k_cache.data_ptr()),
+      reinterpret_cast<const __hip_bfloat16*>(v_cache.data_ptr()),
+      block_tables.data_ptr<int>(), seq_lens.data_ptr<int>(), (float)scale, nseq,
+      nheads, kvh, (int)v_cache.size(2), head_dim, block_size, max_blocks, npart,
+      (int)chunk, current_stream());
+}
+
 }  // namespace
 
 void register_attention_ops(pybind11::module& m) {
+  m.def("chunk_attention_prefill", &chunk_attention_prefill,
+        "paged chunk-masked prefill attention, f32 out (CDNA4)");
+  m.def("chunk_attention_decode", &chunk_attention_decode,
+        "paged chunk-masked decode attention, f32 out (CDNA4)");
   m.def("windowed_attention_prefill", &windowed_attention_prefill,
         "paged windowed prefill attention with a softmax sink (CDNA4)");
   m.def("windowed_attention_decode", &windowed_attention_decode,

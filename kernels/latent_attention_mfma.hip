@@ -388,7 +388,8 @@ int latent_decode_num_splits(int nseq, int heads, int max_keys) {
 
 #define LM_SHAPES(X) \
   X(2, 2) X(2, 3) X(4, 3) X(4, 4) X(6, 4) X(6, 5) X(8, 5) X(8, 6) X(16, 9) \
-  X(16, 10) X(32, 17) X(32, 18)
+  X(16, 10) X(32, 17) X(32, 18)                                             \
+  /* no rotated part */ X(2, 1) X(4, 2) X(8, 4) X(16, 8) X(32, 16)
 
 bool latent_prefill_mfma_usable(int rank, int rot, int block_size) {
   (void)block_size;

@@ -110,6 +110,7 @@ def _paged(ctx_lens, kv_heads, v_heads, dim, vdim, bs, dtype, g):
 @pytest.mark.parametrize("chunk", [0, 5, 16, 300])
 @pytest.mark.parametrize("heads,kv_heads,v_heads,dim,vdim", [
     (8, 2, 1, 16, 24), (4, 4, 2, 64, 64), (6, 2, 2, 40, 300),
+    (8, 4, 2, 128, 128), (16, 2, 1, 128, 128), (4, 2, 1, 64, 64),   # matrix-core shapes
 ])
 def test_chunk_attention(dtype, chunk, heads, kv_heads, v_heads, dim, vdim):
     g = torch.Generator().manual_seed(11)
@@ -133,6 +134,24 @@ def test_chunk_attention(dtype, chunk, heads, kv_heads, v_heads, dim, vdim):
     ops.chunk_attention_decode(q1.to(DEV), kc.to(DEV), vc.to(DEV), tables.to(DEV),
                                _i32(ctx1).to(DEV), 0.3, chunk, out)
     _close(out, want, dtype, "single queries")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("chunk", [0, 64, 100, 257, 1000])
+@pytest.mark.parametrize("new,ctx", [([300, 40], [330, 700]), ([513], [513]), ([2, 260], [130, 261])])
+def test_chunk_attention_long_portions(dtype, chunk, new, ctx):
+    """Portions that span several query and key tiles of the matrix-core
+    kernel, chunk edges inside tiles and on their borders."""
+    heads, kv_heads, v_heads, dim = 4, 2, 1, 128
+    g = torch.Generator().manual_seed(12)
+    kc, vc, tables = _paged(ctx, kv_heads, v_heads, dim, dim, 16, dtype, g)
+    qsl = _i32([0] + torch.tensor(new).cumsum(0).tolist())
+    q = torch.randn(sum(new), heads, dim, generator=g).to(dtype)
+    want = ref.chunk_attention(q, kc, vc, tables, qsl, _i32(ctx), 0.1, chunk)
+    out = torch.empty(sum(new), heads, dim, dtype=torch.float32, device=DEV)
+    ops.chunk_attention_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), tables.to(DEV),
+                                qsl.to(DEV), _i32(ctx).to(DEV), 0.1, max(new), chunk, out)
+    _close(out, want, dtype, "portions")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

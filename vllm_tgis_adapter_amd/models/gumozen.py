@@ -140,11 +140,23 @@ def model_config_from_json(model: str, hf: dict) -> ModelConfig:
 
 def native_extensions(cfg: ModelConfig) -> list[str]:
     """Stream ops, token shift, norm + rotation + cache write, chunk-masked
-    attention, the recurrence, gates and router live in the sequence
-    extension; latent attention has its own."""
+    attention of any shape, the recurrence, gates and router live in the
+    sequence extension; latent attention has its own; an attention mixer whose
+    shape the matrix-core kernels take needs the attention extension too."""
     need = ["_C_seq"]
-    if any(e.get("type") == "latent_attention" for e in cfg.hf_config["layers"]):
+    layers = cfg.hf_config["layers"]
+    if any(e.get("type") == "latent_attention" for e in layers):
         need.append("_C_lat")
+    for e in layers:
+        if e.get("type") != "attention":
+            continue
+        m = e["mixer"]
+        dim = int(m["dim"])
+        if ops.chunk_attention_uses_matrix_cores(
+                cfg.dtype, int(m["heads"]), int(m.get("kv_heads", m["heads"])), dim,
+                int(m.get("vdim", dim))):
+            need.append("_C_attn")
+            break
     return need
 
 

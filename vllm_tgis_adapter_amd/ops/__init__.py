@@ -1086,6 +1086,27 @@ def qk_norm_rope_cache_write(q, k, v, q_weight, k_weight, eps, positions, inv_fr
                                               slot_mapping)
 
 
+def _chunk_matrix_core_fits(q, k_cache, v_cache, out, single: bool) -> bool:
+    """The chunk variants of the MFMA kernels take bf16, equal key and value
+    size of 128 (single queries: also 64), up to 8 query heads per key head, a
+    whole number of key heads per value head, f32 output."""
+    if _attn_ext() is None or _FORCE_REFERENCE or q.dtype != torch.bfloat16:
+        return False
+    d = q.shape[-1]
+    kvh, vh = k_cache.shape[2], v_cache.shape[2]
+    group = q.shape[1] // kvh
+    return (d in ((64, 128) if single else (128,)) and v_cache.shape[-1] == d
+            and 1 <= group <= 8 and q.shape[1] == group * kvh and kvh % vh == 0
+            and q.is_contiguous() and out.is_contiguous())
+
+
+def chunk_attention_uses_matrix_cores(dtype: torch.dtype, heads: int, kv_heads: int,
+                                      dim: int, vdim: int) -> bool:
+    """Shape test of the above without tensors (which extensions a model needs)."""
+    return (dtype == torch.bfloat16 and dim == vdim and dim in (64, 128)
+            and heads % kv_heads == 0 and 1 <= heads // kv_heads <= 8)
+
+
 def chunk_attention_prefill(q, k_cache, v_cache, block_tables, query_start_loc,
                             seq_lens, scale, max_query_len, chunk: int,
                             out: torch.Tensor) -> torch.Tensor:
@@ -1095,6 +1116,11 @@ def chunk_attention_prefill(q, k_cache, v_cache, block_tables, query_start_loc,
     hold fewer heads than the key cache (key head g reads value head g mod
     Gv).  out [T, H, vdim] f32."""
     if q.numel() and _native_seq(q):
+        if _chunk_matrix_core_fits(q, k_cache, v_cache, out, single=False):
+            _attn_ext().chunk_attention_prefill(
+                out, q, k_cache, v_cache, block_tables, query_start_loc, seq_lens,
+                float(scale), int(max_query_len), int(chunk))
+            return out
         _S.chunk_attention(out, q, k_cache, v_cache, block_tables, query_start_loc,
                            seq_lens, float(scale), int(max_query_len), int(chunk))
         return out
@@ -1107,6 +1133,10 @@ def chunk_attention_decode(q, k_cache, v_cache, block_tables, seq_lens, scale,
                            chunk: int, out: torch.Tensor) -> torch.Tensor:
     """Same attention for one new query per sequence (length 0 = padding row)."""
     if q.numel() and _native_seq(q):
+        if _chunk_matrix_core_fits(q, k_cache, v_cache, out, single=True):
+            _attn_ext().chunk_attention_decode(out, q, k_cache, v_cache, block_tables,
+                                               seq_lens, float(scale), int(chunk))
+            return out
         _S.chunk_attention(out, q, k_cache, v_cache, block_tables, None, seq_lens,
                            float(scale), 1, int(chunk))
         return out
