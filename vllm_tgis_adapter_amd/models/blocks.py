@@ -1120,8 +1120,11 @@ class GatedRoutedExperts(nn.Module):
             else:
                 self.down.data[:, e * ff:(e + 1) * ff].copy_(d.to(self.dtype))
 
-    def forward(self, h: torch.Tensor) -> torch.Tensor:
-        z = torch.nn.functional.linear(h.float(), self.router)
+    def forward(self, h: torch.Tensor, router_in: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``router_in``: the f32 rows h was rounded from, when the caller has
+        them; the router then reads those instead of the rounded copy."""
+        z = torch.nn.functional.linear(h.float() if router_in is None else router_in,
+                                       self.router)
         dense, ids, w = ops.moe_route_sigmoid(z, self.top)
         ne = self.experts
         if not self.grouped:

@@ -202,7 +202,8 @@ class GumozenLayer(nn.Module):
             return
         h = ops.stream_add_rms_norm(x, y, self.norm1, self.eps, 1.0, layer_scale=self.ls1,
                                     cast_dtype=self.dtype)
-        ops.stream_add_rms_norm(x, self.mlp(h), self.norm2, self.eps, 1.0,
+        # the router reads the f32 stream itself, the experts its rounded copy
+        ops.stream_add_rms_norm(x, self.mlp(h, router_in=x), self.norm2, self.eps, 1.0,
                                 layer_scale=self.ls2)
 
 
