@@ -210,15 +210,24 @@ __global__ __launch_bounds__(256) void matrix_scan_kernel(ScanArgs a) {
   const KQ* kp = reinterpret_cast<const KQ*>(a.k) + (long)grp * a.nk;
   const T* vp = reinterpret_cast<const T*>(a.v) + (long)h * a.vdim;
 
+  // the next row's inputs are loaded while this row is computed: with two
+  // waves per SIMD the load latency is otherwise paid once per token
+  float kk[NPT], qq[NPT], vj[VPT];
+  float4 gt;
+  auto load_row = [&](long row, float* k_, float* q_, float* v_, float4& g_) {
+    load_slice<KQ>(kp + row * a.k_st, n0, a.nk, vec, k_);
+    load_slice<KQ>(qp + row * a.q_st, n0, a.nk, vec, q_);
+#pragma unroll
+    for (int c = 0; c < VPT; ++c) v_[c] = ScalarOps<T>::to_f32(vp[row * a.v_st + jc[c]]);
+    g_ = KIND == KIND_HGRN2 ? make_float4(0.f, 0.f, 0.f, 0.f) : gp[row * a.heads];
+  };
+  load_row(row0, kk, qq, vj, gt);
   for (int r = 0; r < n; ++r) {
     const long row = row0 + r;
-    float kk[NPT], qq[NPT], vj[VPT];
-    load_slice<KQ>(kp + row * a.k_st, n0, a.nk, vec, kk);
-    load_slice<KQ>(qp + row * a.q_st, n0, a.nk, vec, qq);
-#pragma unroll
-    for (int c = 0; c < VPT; ++c) vj[c] = ScalarOps<T>::to_f32(vp[row * a.v_st + jc[c]]);
-    const float4 gt = KIND == KIND_HGRN2 ? make_float4(0.f, 0.f, 0.f, 0.f)
-                                         : gp[row * a.heads];
+    float kn[NPT], qn[NPT], vn[VPT];
+    float4 gn;
+    const bool more = r + 1 < n;       // uniform over the workgroup
+    if (more) load_row(row + 1, kn, qn, vn, gn);
     const float alpha = gt.x, beta = gt.y;
     float dot[VPT], ndot = 0.f;
 #pragma unroll
@@ -248,6 +257,13 @@ __global__ __launch_bounds__(256) void matrix_scan_kernel(ScanArgs a) {
       const float yv = KIND == KIND_MLSTM ? d * den : d + c2 * vj[c];
       if (ns == 0 && jbase + c < a.vdim)
         a.y[row * a.y_st + (long)h * a.vdim + jbase + c] = yv;
+    }
+    if (more) {
+#pragma unroll
+      for (int i = 0; i < NPT; ++i) { kk[i] = kn[i]; qq[i] = qn[i]; }
+#pragma unroll
+      for (int c = 0; c < VPT; ++c) vj[c] = vn[c];
+      gt = gn;
     }
   }
 

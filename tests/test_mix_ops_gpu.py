@@ -61,13 +61,15 @@ def test_token_shift(dtype, width, case):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("pad", [3, 8])      # 8: rows stay 16-byte aligned (vector kernel)
 @pytest.mark.parametrize("heads,kv_heads,v_heads,dim,vdim,rot", [
     (4, 2, 1, 8, 12, 4), (6, 6, 3, 64, 64, 64), (2, 2, 2, 70, 5, 0), (8, 2, 1, 128, 96, 32),
+    (32, 8, 4, 128, 128, 128), (3, 1, 1, 32, 8, 0), (2, 2, 1, 256, 64, 256), (2, 1, 1, 512, 16, 512),
 ])
-def test_qk_norm_rope_cache_write(dtype, heads, kv_heads, v_heads, dim, vdim, rot):
+def test_qk_norm_rope_cache_write(dtype, heads, kv_heads, v_heads, dim, vdim, rot, pad):
     g = torch.Generator().manual_seed(3)
     t, bs, blocks = 9, 4, 6
-    cols = heads * dim + kv_heads * dim + v_heads * vdim + 3
+    cols = heads * dim + kv_heads * dim + v_heads * vdim + pad
     proj = torch.randn(t, cols, generator=g).to(dtype)
     a, b = heads * dim, (heads + kv_heads) * dim
     c = b + v_heads * vdim
@@ -155,7 +157,7 @@ def test_chunk_attention_long_portions(dtype, chunk, new, ctx):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,vdim,gate", [(3, 10, True), (4, 64, True), (2, 200, False)])
+@pytest.mark.parametrize("heads,vdim,gate", [(3, 10, True), (4, 64, True), (2, 200, False), (2, 300, True)])
 def test_diff_combine(dtype, heads, vdim, gate):
     g = torch.Generator().manual_seed(5)
     t = 11
@@ -171,7 +173,7 @@ def test_diff_combine(dtype, heads, vdim, gate):
 @pytest.mark.parametrize("in_dtype,out_dtype", [
     (torch.float32, torch.float32), (torch.float32, torch.bfloat16),
     (torch.bfloat16, torch.bfloat16)])
-@pytest.mark.parametrize("groups,gsize", [(1, 80), (4, 64), (3, 7), (2, 300)])
+@pytest.mark.parametrize("groups,gsize", [(1, 80), (4, 64), (3, 7), (2, 300), (1, 1536), (2, 256)])
 def test_group_rms_norm(in_dtype, out_dtype, groups, gsize):
     g = torch.Generator().manual_seed(6)
     y = (torch.randn(7, groups * gsize, generator=g) * 3).to(in_dtype)

@@ -961,8 +961,11 @@ class DiffAttention(_Mixer):
         self.heads, self.kv_heads, self.dim, self.vdim = heads, kv_heads, dim, vdim
         self.scale, self.diff, self.eps, self.chunk = scale, diff, eps, chunk
         self.rot_dims, self.head_gate = rot_dims, head_gate
-        self.in_rows = (2 * heads * dim + 2 * kv_heads * dim + kv_heads * vdim
-                        + (heads if head_gate else 0))
+        rows = 2 * heads * dim + 2 * kv_heads * dim + kv_heads * vdim + (heads if head_gate else 0)
+        # zero rows behind the gate keep every projected row 16-byte aligned,
+        # which the vector kernels ask for
+        self.pad_rows = -rows % 8
+        self.in_rows = rows + self.pad_rows
         self.out_rows = heads * vdim
         self._alloc(width, own_in, dtype)
         self.q_norm = _f32_param(dim, fill=1.0)
@@ -982,8 +985,9 @@ class DiffAttention(_Mixer):
         for w in [q, k, t["v"]] + ([t["g"]] if self.head_gate else []):
             weight[off:off + w.shape[0]].copy_(w.to(weight.dtype))
             off += w.shape[0]
-        if off != self.in_rows:
+        if off != self.in_rows - self.pad_rows:
             raise ValueError("projection tensors do not add up to the mixer's rows")
+        weight[off:].zero_()
 
     def load_rest(self, t) -> None:
         import math
@@ -1020,7 +1024,7 @@ class DiffAttention(_Mixer):
                 q[npt:], k_cache, v_cache, meta.decode_block_tables,
                 meta.decode_seq_lens, self.scale, self.chunk, out=maps[npt:])
         return ops.diff_combine(maps.view(t, 2, nh, dv), self.lam, 1.0 - self.diff, self.eps,
-                                proj[:, c:] if self.head_gate else None, self.dtype)
+                                proj[:, c:c + nh] if self.head_gate else None, self.dtype)
 
 
 class HGRN2Mixer(_Mixer):
