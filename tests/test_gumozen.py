@@ -307,8 +307,11 @@ def test_routed_experts_alone(device):
         mod = blocks.GatedRoutedExperts(width, experts=experts, top=top, ff=ff,
                                         dtype=torch.float32)
         mod.load(router, [e[0] for e in ex], [e[1] for e in ex], [e[2] for e in ex])
-        _close(mod.to(device)(h.to(device)).double().cpu(), want,
-               what=f"experts {experts} top {top}")
+        mod = mod.to(device)
+        _close(mod(h.to(device)).double().cpu(), want, what=f"experts {experts} top {top}")
+        # the router may be fed the rows the experts' input was rounded from
+        _close(mod(h.to(device), router_in=h.to(device)).double().cpu(), want,
+               what="router fed separately")
 
 
 def test_weight_on_the_input_is_not_weight_on_the_output():
